@@ -18,6 +18,9 @@ void rms_norm_rows(bool bf16, const float* x, const void* w, int nw, float* h, v
                    hipStream_t st);
 // x += y / sqrt(mean(y^2) + eps) * w; xa: x in the activation type (bf16 only, may be null)
 void add_rms_norm(bool bf16, float* x, const void* y, const void* w, void* xa, int T, int W, float eps, hipStream_t st);
+// x += y (y in the activation type, may be null), then out = x / sqrt(mean(x^2) + eps) * w in the activation type
+void add_rms_norm_rows(bool bf16, float* x, const void* y, const void* w, void* out, int T, int W, float eps,
+                       hipStream_t st);
 // x += s1 * y1 + s2 * (y2 + y3); s1, s2 f32 [W] or null; y2 f32 when y2_f32 else activation type; y2, y3 may be null
 void residual_add_scaled(bool bf16, float* x, const void* y1, const float* s1, const void* y2, bool y2_f32,
                          const void* y3, const float* s2, void* xa, int64_t T, int W, hipStream_t st);

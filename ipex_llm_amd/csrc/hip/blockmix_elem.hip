@@ -74,6 +74,26 @@ __global__ void __launch_bounds__(1024) add_rms_norm_k(float* __restrict__ x, co
   }
 }
 
+// x += y (y may be null), then out = x / sqrt(mean(x^2) + eps) * w: one sublayer's residual sum and the next norm
+template <typename E>
+__global__ void __launch_bounds__(1024) add_rms_norm_rows_k(float* __restrict__ x, const E* __restrict__ y,
+                                                          const E* __restrict__ w, E* __restrict__ out, int W, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * W;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = xr[c];
+    if (y) {
+      v += ldf(y + t * W + c);
+      xr[c] = v;
+    }
+    q += v * v;
+  }
+  const float rs = 1.0f / sqrtf(block_sum(q, red) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stf(out + t * W + c, xr[c] * rs * ldf(w + c));   // own writes
+}
+
 template <typename E>
 __global__ void __launch_bounds__(256) residual_add_scaled_k(float* __restrict__ x, const E* __restrict__ y1,
                                                             const float* __restrict__ s1, const void* __restrict__ y2,
@@ -262,6 +282,15 @@ void add_rms_norm(bool bf16, float* x, const void* y, const void* w, void* xa, i
   if (T <= 0) return;
   if (bf16) add_rms_norm_k<__bf16><<<T, row_threads(W, T), 0, st>>>(x, (const __bf16*)y, (const __bf16*)w, (__bf16*)xa, W, eps);
   else add_rms_norm_k<float><<<T, row_threads(W, T), 0, st>>>(x, (const float*)y, (const float*)w, nullptr, W, eps);
+}
+
+void add_rms_norm_rows(bool bf16, float* x, const void* y, const void* w, void* out, int T, int W, float eps,
+                       hipStream_t st) {
+  if (T <= 0) return;
+  if (bf16)
+    add_rms_norm_rows_k<__bf16><<<T, row_threads(W, T), 0, st>>>(x, (const __bf16*)y, (const __bf16*)w, (__bf16*)out, W, eps);
+  else
+    add_rms_norm_rows_k<float><<<T, row_threads(W, T), 0, st>>>(x, (const float*)y, (const float*)w, (float*)out, W, eps);
 }
 
 void residual_add_scaled(bool bf16, float* x, const void* y1, const float* s1, const void* y2, bool y2_f32,

@@ -30,16 +30,17 @@ void latent_kv_store(bool bf16, const void* dkv, int64_t ld, const void* norm_w,
 int latent_attention_plan(bool bf16, int H, int r, int dr, int* kt, int* nw, int* hb);
 // key splits (grid z) for T query tokens whose longest context is max_ctx
 int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx);
-// part: f32 scratch [T, H, nsplit, r + 2] when nsplit > 1
+// part: f32 scratch [T, H, nsplit, r + 2] when nsplit > 1; window > 0: only the keys pos - window < j <= pos count
 void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t qr_st, int64_t qr_sh, const void* rows,
                       int bs, const int32_t* block_tables, int bt_width, const int32_t* seq_of, const int64_t* pos,
                       float scale, const void* gate, int64_t g_st, void* out, float* part, int nsplit, int T, int H,
-                      int r, int dr, hipStream_t st);
+                      int r, int dr, int window, hipStream_t st);
 
-// causal softmax of f32 score rows [R, L] (row stride ld), row i -> position pos[i / H]; bf16: weights leave
-// as hi + lo bf16 pairs (same row stride), f32 (hi == null): in place
+// causal softmax of f32 score rows [R, L] (row stride ld), row i -> position pos[i / H], column j -> key key0 + j,
+// window > 0: only the keys pos - window < key <= pos count; bf16: weights leave as hi + lo bf16 pairs (same row
+// stride), f32 (hi == null): in place
 void causal_softmax(bool bf16, float* sc, int64_t ld, const int64_t* pos, int H, float scale, int64_t R, int L, void* hi,
-                    void* lo, hipStream_t st);
+                    void* lo, int64_t key0, int window, hipStream_t st);
 
 // q, k [T, H, d], v [T, H, dv], gate pre-activations [T, H]: rows of *_ld elements
 void mlstm_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
@@ -49,6 +50,8 @@ void mlstm_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k
 void head_rms_gate(bool bf16, const float* h, const void* norm_w, const void* gate, int64_t g_ld, void* out, int T,
                    int H, int dv, float eps, hipStream_t st);
 void glu_gelu(bool bf16, const void* gu, void* out, int64_t T, int64_t I, hipStream_t st);
+// act(gate) * up; act 0: tanh-GELU, 1: ReLU, 2: SiLU
+void glu_act(bool bf16, const void* gu, void* out, int64_t T, int64_t I, int act, hipStream_t st);
 
 }  // namespace sm
 }  // namespace illm

@@ -202,7 +202,7 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
                                                     const int32_t* __restrict__ seq_of, const int64_t* __restrict__ pos,
                                                     float scale, const E* __restrict__ gate, int64_t g_st,
                                                     E* __restrict__ out, float* __restrict__ part, int H, int r, int dr,
-                                                    int KT, int DP) {
+                                                    int KT, int DP, int window) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int D = r + dr, D4 = (D + 3) & ~3;
   const int nsplit = gridDim.z, zs = blockIdx.z;
@@ -246,6 +246,9 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
   const int64_t p = pos[t];
   const int32_t* tab = bt + (int64_t)seq_of[t] * bt_w;
   const int ntiles = (int)(p / KT) + 1;
+  // a window keeps the keys p - window < j <= p: tiles before the first of them are skipped
+  const int64_t lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  const int tile0 = (int)(lo / KT);
   float m[HB], l[HB], o[HB][RC];
 #pragma unroll
   for (int h = 0; h < HB; h++) {
@@ -254,7 +257,7 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
 #pragma unroll
     for (int c = 0; c < RC; c++) o[h][c] = 0.f;
   }
-  for (int ti = zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
+  for (int ti = tile0 + zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
     const int64_t k0 = (int64_t)ti * KT;
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
@@ -292,7 +295,7 @@ __global__ void __launch_bounds__(256) latent_attn_k(const E* __restrict__ q_lat
     for (int h = 0; h < HB; h++) s[h] = 0.f;
     // 64 / KT lanes share a key: each takes a slice of the r + dr products, summed by lane exchange
     const int kj = lane & (KT - 1), grp = lane / KT, G = 64 / KT;
-    const bool valid = kj < nvalid;
+    const bool valid = kj < nvalid && k0 + kj >= lo;
     if (valid) {
       const E* kr = kt + kj * DP;
       const int steps = D4 >> 2;
@@ -406,7 +409,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_k(const __bf16* __restri
                                                          const int64_t* __restrict__ pos, float scale,
                                                          const __bf16* __restrict__ gate, int64_t g_st,
                                                          __bf16* __restrict__ out, float* __restrict__ part, int H, int r,
-                                                         int dr, int DP) {
+                                                         int dr, int DP, int window) {
   typedef __bf16 E;
   constexpr int KT = 16;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -449,13 +452,16 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_k(const __bf16* __restri
   const int64_t p = pos[t];
   const int32_t* tab = bt + (int64_t)seq_of[t] * bt_w;
   const int ntiles = (int)(p / KT) + 1;
+  // a window keeps the keys p - window < j <= p: tiles before the first of them are skipped
+  const int64_t lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  const int tile0 = (int)(lo / KT);
   float m_r = -INFINITY, l_r = 0.f;                                // of head r16 (the same in its four lanes)
   float o[HB][RC];
 #pragma unroll
   for (int h = 0; h < HB; h++)
 #pragma unroll
     for (int c = 0; c < RC; c++) o[h][c] = 0.f;
-  for (int ti = zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
+  for (int ti = tile0 + zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
     const int64_t k0 = (int64_t)ti * KT;
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
@@ -499,7 +505,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_k(const __bf16* __restri
     float sv[4], mloc = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      sv[i] = (4 * g + i) < nvalid ? acc[i] * scale : -INFINITY;
+      sv[i] = (4 * g + i) < nvalid && k0 + 4 * g + i >= lo ? acc[i] * scale : -INFINITY;
       mloc = fmaxf(mloc, sv[i]);
     }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
@@ -621,28 +627,31 @@ __global__ void __launch_bounds__(128) latent_attn_combine_k(const float* __rest
 // carry the weights to ~2^-17 instead of 2^-9.
 template <typename E>
 __global__ void __launch_bounds__(256) causal_softmax_k(float* __restrict__ sc, int64_t ld, const int64_t* __restrict__ pos,
-                                                       int H, float scale, int L, E* __restrict__ hi, E* __restrict__ lo) {
+                                                       int H, float scale, int L, E* __restrict__ hi, E* __restrict__ lo,
+                                                       int64_t key0, int window) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
   const int64_t p = pos[row / H];
-  const int nk = (int)min((int64_t)L, p + 1);
+  // column j is key key0 + j; visible: key <= p, and key > p - window with a window
+  const int nk = (int)max((int64_t)0, min((int64_t)L, p - key0 + 1));
+  const int j0 = window > 0 ? (int)max((int64_t)0, min((int64_t)nk, p - window + 1 - key0)) : 0;
   float* s = sc + row * ld;
   float mx = -INFINITY;
-  for (int j = threadIdx.x; j < nk; j += blockDim.x) mx = fmaxf(mx, s[j] * scale);
+  for (int j = j0 + threadIdx.x; j < nk; j += blockDim.x) mx = fmaxf(mx, s[j] * scale);
   mx = wave_max(mx);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
   __syncthreads();
   for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
   float sum = 0.f;
-  for (int j = threadIdx.x; j < nk; j += blockDim.x) {
+  for (int j = j0 + threadIdx.x; j < nk; j += blockDim.x) {
     const float e = expf(s[j] * scale - mx);
     s[j] = e;
     sum += e;
   }
   const float inv = 1.0f / block_sum(sum, red);
   for (int j = threadIdx.x; j < L; j += blockDim.x) {
-    const float w = j < nk ? s[j] * inv : 0.f;
+    const float w = j >= j0 && j < nk ? s[j] * inv : 0.f;
     if (hi) {
       const E h = (E)w;
       hi[row * ld + j] = h;
@@ -856,6 +865,20 @@ __global__ void __launch_bounds__(256) glu_gelu_k(const E* __restrict__ gu, E* _
   stf(out + i, a * u);
 }
 
+// act(gate) * up; ACT 0: tanh-GELU, 1: ReLU, 2: SiLU (f32 math)
+template <typename E, int ACT>
+__global__ void __launch_bounds__(256) glu_act_k(const E* __restrict__ gu, E* __restrict__ out, int64_t T, int64_t I) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= T * I) return;
+  const int64_t t = i / I, c = i - t * I;
+  const float g = ldf(gu + t * 2 * I + c), u = ldf(gu + t * 2 * I + I + c);
+  float a;
+  if (ACT == 1) a = fmaxf(g, 0.f);
+  else if (ACT == 2) a = g / (1.0f + expf(-g));
+  else a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  stf(out + i, a * u);
+}
+
 }  // namespace
 
 #define SM_DISPATCH(bf16, ...)                 \
@@ -957,7 +980,7 @@ static const bool kUseMfma = []() {
   return !(e && e[0] == '0');
 }();
 
-int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx) {
+int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx) {   // with a window: the keys it spans
   int KT = 0, NW = 0, hb = 8;
   if (bf16 && kUseMfma && latent_attention_plan_mfma(H, r, dr, &NW, &hb) > 0) KT = 16;
   else if (latent_attention_plan(bf16, H, r, dr, &KT, &NW, &hb) < 0) return 1;
@@ -971,7 +994,7 @@ int latent_attention_splits(bool bf16, int T, int H, int r, int dr, int max_ctx)
 void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t qr_st, int64_t qr_sh, const void* rows,
                       int bs, const int32_t* block_tables, int bt_width, const int32_t* seq_of, const int64_t* pos,
                       float scale, const void* gate, int64_t g_st, void* out, float* part, int nsplit, int T, int H,
-                      int r, int dr, hipStream_t st) {
+                      int r, int dr, int window, hipStream_t st) {
   if (T <= 0) return;
   const int rc = (r + 63) / 64;
   int KT = 0, NW = 0, hb = 8;
@@ -983,7 +1006,7 @@ void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t q
 #define SM_ATTN_M(RC, HBV)                                                                                            \
   hipLaunchKernelGGL((latent_attn_mfma_k<RC, HBV>), grid, block, lds, st, (const __bf16*)q_lat, (const __bf16*)q_rot,  \
                      qr_st, qr_sh, (const __bf16*)rows, bs, block_tables, bt_width, seq_of, pos, scale,                \
-                     (const __bf16*)gate, g_st, (__bf16*)out, part, H, r, dr, DP)
+                     (const __bf16*)gate, g_st, (__bf16*)out, part, H, r, dr, DP, window)
       if (hb == 8) {
         if (rc <= 1) { SM_ATTN_M(1, 8); }
         else if (rc <= 2) { SM_ATTN_M(2, 8); }
@@ -1007,7 +1030,8 @@ void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t q
 #define SM_ATTN(RC, HBV)                                                                                              \
   SM_DISPATCH(bf16, hipLaunchKernelGGL((latent_attn_k<E, RC, HBV>), grid, block, lds, st, (const E*)q_lat,             \
                                        (const E*)q_rot, qr_st, qr_sh, (const E*)rows, bs, block_tables, bt_width,      \
-                                       seq_of, pos, scale, (const E*)gate, g_st, (E*)out, part, H, r, dr, KT, DP))
+                                       seq_of, pos, scale, (const E*)gate, g_st, (E*)out, part, H, r, dr, KT, DP,      \
+                                       window))
   if (hb == 8) {
     if (rc <= 1) { SM_ATTN(1, 8); }
     else if (rc <= 2) { SM_ATTN(2, 8); }
@@ -1025,14 +1049,14 @@ void latent_attention(bool bf16, const void* q_lat, const void* q_rot, int64_t q
 }
 
 void causal_softmax(bool bf16, float* sc, int64_t ld, const int64_t* pos, int H, float scale, int64_t R, int L, void* hi,
-                    void* lo, hipStream_t st) {
+                    void* lo, int64_t key0, int window, hipStream_t st) {
   if (R <= 0 || L <= 0) return;
   if (bf16) {
     hipLaunchKernelGGL(causal_softmax_k<__bf16>, dim3((unsigned)R), dim3(256), 0, st, sc, ld, pos, H, scale, L,
-                       (__bf16*)hi, (__bf16*)lo);
+                       (__bf16*)hi, (__bf16*)lo, key0, window);
   } else {
     hipLaunchKernelGGL(causal_softmax_k<float>, dim3((unsigned)R), dim3(256), 0, st, sc, ld, pos, H, scale, L,
-                       (float*)nullptr, (float*)nullptr);
+                       (float*)nullptr, (float*)nullptr, key0, window);
   }
 }
 
@@ -1067,6 +1091,19 @@ void head_rms_gate(bool bf16, const float* h, const void* norm_w, const void* ga
   if (T <= 0) return;
   SM_DISPATCH(bf16, hipLaunchKernelGGL(head_rms_gate_k<E>, dim3(T, H), dim3(64), 0, st, h, (const E*)norm_w,
                                        (const E*)gate, g_ld, (E*)out, H, dv, eps));
+}
+
+void glu_act(bool bf16, const void* gu, void* out, int64_t T, int64_t I, int act, hipStream_t st) {
+  const int64_t n = T * I;
+  if (n <= 0) return;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (act == 1) {
+    SM_DISPATCH(bf16, hipLaunchKernelGGL((glu_act_k<E, 1>), dim3(blocks), dim3(256), 0, st, (const E*)gu, (E*)out, T, I));
+  } else if (act == 2) {
+    SM_DISPATCH(bf16, hipLaunchKernelGGL((glu_act_k<E, 2>), dim3(blocks), dim3(256), 0, st, (const E*)gu, (E*)out, T, I));
+  } else {
+    SM_DISPATCH(bf16, hipLaunchKernelGGL((glu_act_k<E, 0>), dim3(blocks), dim3(256), 0, st, (const E*)gu, (E*)out, T, I));
+  }
 }
 
 void glu_gelu(bool bf16, const void* gu, void* out, int64_t T, int64_t I, hipStream_t st) {

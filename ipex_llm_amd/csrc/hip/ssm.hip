@@ -1,0 +1,272 @@
+// Kernels of the state-space mixer (gfx950, wave64).
+//
+//   conv + SiLU        a thread per (token, channel); tokens before a portion's
+//                      start come from the sequence's state slot, positions
+//                      before 0 are zero; a second launch (or the same one at
+//                      decode) leaves the portion's last inputs in the slot
+//   selective scan     S' = a S + dt B x^T, y = S'^T C + D x.  One workgroup:
+//                      64 value columns of one (sequence, head).  Wave w keeps
+//                      the state rows [w NS, (w + 1) NS) of those columns in
+//                      registers; tokens go through LDS in chunks (B and C
+//                      rows zero padded to the waves' rows, the step sizes with
+//                      their softplus and the decays computed once per chunk);
+//                      every wave leaves a partial y per token and the partials
+//                      are summed in a fixed order, so a result never depends
+//                      on how the tokens were cut into steps
+//   gated group norm   y silu(z), every group divided by its root mean square
+//
+// Activations are bf16 or f32 (template E); accumulation is always f32.
+#include "ssm.h"
+
+#include <math.h>
+
+namespace illm {
+namespace ssm {
+namespace {
+
+template <typename E> __device__ __forceinline__ float ldf(const E* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<__bf16>(const __bf16* p) { return (float)*p; }
+template <typename E> __device__ __forceinline__ void stf(E* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<__bf16>(__bf16* p, float v) { *p = (__bf16)v; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < nw; i++) s += red[i];
+  return s;
+}
+__device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
+
+constexpr int kMaxTaps = 16;
+
+// ------------------------------------------------------------------ convolution
+template <typename E>
+__global__ void __launch_bounds__(256) conv_silu_k(const E* __restrict__ u, int64_t u_ld, const float* __restrict__ w,
+                                                  const float* __restrict__ bias, int taps, float* __restrict__ state,
+                                                  const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_of,
+                                                  const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
+                                                  float* __restrict__ out, int C, bool single) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int b = seq_of[t];
+  const int i = t - cu[b];                                          // index inside the portion
+  const int64_t p = pos[t];
+  float* st = state + (int64_t)slots[b] * (taps - 1) * C + c;       // [taps - 1][C], oldest first
+  float acc = bias[c];
+  float hist[kMaxTaps];                                             // inputs of positions p - taps + 1 .. p
+  for (int j = 0; j < taps; j++) {
+    const int back = taps - 1 - j;
+    float v = 0.f;
+    if (back <= i) v = ldf(u + (int64_t)(t - back) * u_ld + c);
+    else if (p - back >= 0) v = st[(int64_t)(taps - 1 + i - back) * C];
+    hist[j] = v;
+    acc = fmaf(w[(int64_t)c * taps + j], v, acc);
+  }
+  out[(int64_t)t * C + c] = silu(acc);
+  if (single)                                                       // the only token of its sequence: advance the state
+    for (int j = 1; j < taps; j++) st[(int64_t)(j - 1) * C] = hist[j];
+}
+
+// after a portion of n tokens that started at position p0: the slot holds the inputs of positions p0 + n - taps + 1 ..
+// p0 + n - 1 (zeros for positions before 0)
+template <typename E>
+__global__ void __launch_bounds__(256) conv_state_k(const E* __restrict__ u, int64_t u_ld, int taps,
+                                                   float* __restrict__ state, const int32_t* __restrict__ cu,
+                                                   const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
+                                                   int C) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  if (n <= 0) return;
+  const int64_t p0 = pos[t0];
+  float* st = state + (int64_t)slots[b] * (taps - 1) * C + c;
+  float nv[kMaxTaps];
+  for (int k = 0; k < taps - 1; k++) {
+    const int64_t i = (int64_t)n - (taps - 1) + k;                  // index inside the portion of that position
+    float v = 0.f;
+    if (i >= 0) v = ldf(u + (int64_t)(t0 + i) * u_ld + c);
+    else if (p0 + i >= 0) v = st[(int64_t)(k + n) * C];
+    nv[k] = v;
+  }
+  for (int k = 0; k < taps - 1; k++) st[(int64_t)k * C] = nv[k];
+}
+
+// ------------------------------------------------------------------ scan
+template <typename E, int NS>
+__global__ void __launch_bounds__(NS == 64 ? 1024 : 256) scan_k(
+    const float* __restrict__ x, int64_t x_ld, const float* __restrict__ Bm, int64_t b_ld, const float* __restrict__ Cm,
+    int64_t c_ld, const E* __restrict__ dtp, int64_t dt_ld, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ S,
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
+    float* __restrict__ out, int H, int P, int G, int N, int TC) {
+  extern __shared__ __align__(16) float sm[];
+  const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * 64;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
+  const int NP = NW * NS;
+  const int t0 = cu[b], n = cu[b + 1] - t0;
+  if (n <= 0) return;
+  const int g = h / (H / G);
+  const int pc = p0 + lane;
+  float* Bs = sm;                                                   // [TC][NP]
+  float* Cs = Bs + (size_t)TC * NP;                                 // [TC][NP]
+  float* xs = Cs + (size_t)TC * NP;                                 // [TC][64]
+  float* pt = xs + (size_t)TC * 64;                                 // [NW][TC][64]
+  float* ds = pt + (size_t)NW * TC * 64;                            // [TC] step sizes, [TC] decays
+  float st[NS];
+  float* Sg = S + (((int64_t)slots[b] * H + h) * N) * P;            // [N][P]
+  const bool fresh = pos[t0] == 0;
+#pragma unroll
+  for (int i = 0; i < NS; i++) {
+    const int nn = wv * NS + i;
+    st[i] = (!fresh && nn < N && pc < P) ? Sg[(int64_t)nn * P + pc] : 0.f;
+  }
+  const float rate = expf(a_log[h]), bias = dt_bias[h], dsk = d_skip[h];
+  for (int c0 = 0; c0 < n; c0 += TC) {
+    const int nt = min(TC, n - c0);
+    __syncthreads();                                                // the last chunk's reads are done
+    for (int i = threadIdx.x; i < nt * NP; i += blockDim.x) {
+      const int tk = i / NP, nn = i - tk * NP;
+      const int64_t t = t0 + c0 + tk;
+      Bs[i] = nn < N ? Bm[t * b_ld + (int64_t)g * N + nn] : 0.f;
+      Cs[i] = nn < N ? Cm[t * c_ld + (int64_t)g * N + nn] : 0.f;
+    }
+    for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
+      const int tk = i >> 6, l = i & 63;
+      xs[i] = p0 + l < P ? x[(int64_t)(t0 + c0 + tk) * x_ld + (int64_t)h * P + p0 + l] : 0.f;
+    }
+    if (threadIdx.x < nt) {
+      const float z = ldf(dtp + (int64_t)(t0 + c0 + threadIdx.x) * dt_ld + h) + bias;
+      const float dt = z > 20.f ? z : log1pf(expf(z));              // softplus
+      ds[threadIdx.x] = dt;
+      ds[TC + threadIdx.x] = expf(-rate * dt);
+    }
+    __syncthreads();
+    for (int tk = 0; tk < nt; tk++) {
+      const float da = ds[TC + tk];
+      const float dx = ds[tk] * xs[tk * 64 + lane];
+      const float4* b4 = (const float4*)(Bs + (size_t)tk * NP + wv * NS);
+      const float4* c4 = (const float4*)(Cs + (size_t)tk * NP + wv * NS);
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < NS / 4; i++) {
+        const float4 bv = b4[i], cv = c4[i];
+        st[4 * i + 0] = fmaf(da, st[4 * i + 0], dx * bv.x);
+        st[4 * i + 1] = fmaf(da, st[4 * i + 1], dx * bv.y);
+        st[4 * i + 2] = fmaf(da, st[4 * i + 2], dx * bv.z);
+        st[4 * i + 3] = fmaf(da, st[4 * i + 3], dx * bv.w);
+        acc = fmaf(st[4 * i + 0], cv.x, acc);
+        acc = fmaf(st[4 * i + 1], cv.y, acc);
+        acc = fmaf(st[4 * i + 2], cv.z, acc);
+        acc = fmaf(st[4 * i + 3], cv.w, acc);
+      }
+      pt[((size_t)wv * TC + tk) * 64 + lane] = acc;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
+      const int tk = i >> 6, l = i & 63;
+      if (p0 + l >= P) continue;
+      float y = 0.f;
+      for (int w = 0; w < NW; w++) y += pt[((size_t)w * TC + tk) * 64 + l];
+      out[((int64_t)(t0 + c0 + tk) * H + h) * P + p0 + l] = fmaf(dsk, xs[i], y);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NS; i++) {
+    const int nn = wv * NS + i;
+    if (nn < N && pc < P) Sg[(int64_t)nn * P + pc] = st[i];
+  }
+}
+
+// ------------------------------------------------------------------ gate + group norm
+template <typename E>
+__global__ void __launch_bounds__(256) gated_group_norm_k(const float* __restrict__ y, const E* __restrict__ z, int64_t z_ld,
+                                                         const E* __restrict__ w, E* __restrict__ out, int C, int gs,
+                                                         float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < gs; c += blockDim.x) {
+    const float v = y[t * C + c0 + c] * silu(ldf(z + t * z_ld + c0 + c));
+    q += v * v;
+  }
+  const float rs = 1.0f / sqrtf(block_sum(q, red) / (float)gs + eps);
+  for (int c = threadIdx.x; c < gs; c += blockDim.x) {
+    const float v = y[t * C + c0 + c] * silu(ldf(z + t * z_ld + c0 + c));
+    stf(out + t * C + c0 + c, v * rs * ldf(w + c0 + c));
+  }
+}
+
+}  // namespace
+
+void conv_silu(bool bf16, const void* u, int64_t u_ld, const float* w, const float* b, int taps, float* state,
+               const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* out, int T,
+               int B, int C, bool single, hipStream_t st) {
+  if (T <= 0 || C <= 0) return;
+  dim3 grid(T, (C + 255) / 256), gs(B, (C + 255) / 256);
+  if (bf16) {
+    conv_silu_k<__bf16><<<grid, 256, 0, st>>>((const __bf16*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C,
+                                              single);
+    if (!single && taps > 1) conv_state_k<__bf16><<<gs, 256, 0, st>>>((const __bf16*)u, u_ld, taps, state, cu, slots, pos, C);
+  } else {
+    conv_silu_k<float><<<grid, 256, 0, st>>>((const float*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C,
+                                             single);
+    if (!single && taps > 1) conv_state_k<float><<<gs, 256, 0, st>>>((const float*)u, u_ld, taps, state, cu, slots, pos, C);
+  }
+}
+
+void selective_scan(bool bf16, const float* x, int64_t x_ld, const float* Bm, int64_t b_ld, const float* Cm,
+                    int64_t c_ld, const void* dt, int64_t dt_ld, const float* dt_bias, const float* a_log,
+                    const float* d_skip, float* S, const int32_t* cu, const int32_t* slots, const int64_t* pos,
+                    float* out, int B, int H, int P, int G, int N, hipStream_t st) {
+  if (B <= 0 || N > kScanMaxState) return;                          // (sizes are refused by the caller beforehand)
+  const int NS = N <= 64 ? 16 : (N <= 128 ? 32 : 64);
+  const int NW = (N + NS - 1) / NS;
+  const int NP = NW * NS;
+  // tokens per chunk: B and C rows, x, the waves' partials and the step sizes within 48 KB
+  int TC = (48 * 1024 / 4) / (2 * NP + 64 + NW * 64 + 2);
+  TC = TC > 16 ? 16 : (TC < 1 ? 1 : TC);
+  const size_t lds = ((size_t)TC * (2 * NP + 64 + NW * 64) + 2 * TC) * sizeof(float);
+  dim3 grid(B, H, (P + 63) / 64), block(64 * NW);
+#define SSM_SCAN(E, NSV)                                                                                              \
+  scan_k<E, NSV><<<grid, block, lds, st>>>(x, x_ld, Bm, b_ld, Cm, c_ld, (const E*)dt, dt_ld, dt_bias, a_log, d_skip, S, \
+                                           cu, slots, pos, out, H, P, G, N, TC)
+  if (bf16) {
+    if (NS == 16) SSM_SCAN(__bf16, 16);
+    else if (NS == 32) SSM_SCAN(__bf16, 32);
+    else SSM_SCAN(__bf16, 64);
+  } else {
+    if (NS == 16) SSM_SCAN(float, 16);
+    else if (NS == 32) SSM_SCAN(float, 32);
+    else SSM_SCAN(float, 64);
+  }
+#undef SSM_SCAN
+}
+
+void gated_group_norm(bool bf16, const float* y, const void* z, int64_t z_ld, const void* w, void* out, int T, int C,
+                      int groups, float eps, hipStream_t st) {
+  if (T <= 0) return;
+  dim3 grid(T, groups);
+  if (bf16)
+    gated_group_norm_k<__bf16><<<grid, 256, 0, st>>>(y, (const __bf16*)z, z_ld, (const __bf16*)w, (__bf16*)out, C,
+                                                     C / groups, eps);
+  else
+    gated_group_norm_k<float><<<grid, 256, 0, st>>>(y, (const float*)z, z_ld, (const float*)w, (float*)out, C, C / groups,
+                                                    eps);
+}
+
+}  // namespace ssm
+}  // namespace illm

@@ -62,6 +62,25 @@ Tensor bm_add_rms_norm(Tensor& x, const Tensor& y, const Tensor& w, double eps, 
   return act_f32 ? x : xa;
 }
 
+Tensor bm_add_rms_norm_rows(Tensor& x, const c10::optional<Tensor>& y, const Tensor& w, double eps, bool act_f32) {
+  c10::DeviceGuard g(x.device());
+  check_f32_rows(x, "bm_add_rms_norm_rows: x f32 [T, W]");
+  const int64_t T = x.size(0), W = x.size(1);
+  const void* yp = nullptr;
+  if (y.has_value() && y->defined()) {
+    TORCH_CHECK(y->is_cuda() && y->scalar_type() == act_type(act_f32) && y->is_contiguous() && y->dim() == 2 &&
+                    y->size(0) == T && y->size(1) == W,
+                "bm_add_rms_norm_rows: y [T, W] in the activation dtype");
+    yp = y->data_ptr();
+  }
+  TORCH_CHECK(w.is_cuda() && w.scalar_type() == act_type(act_f32) && w.is_contiguous() && w.numel() == W,
+              "bm_add_rms_norm_rows: w [W] in the activation dtype");
+  Tensor out = at::empty({T, W}, x.options().dtype(act_type(act_f32)));
+  illm::bm::add_rms_norm_rows(!act_f32, x.data_ptr<float>(), yp, w.data_ptr(), out.data_ptr(), (int)T, (int)W,
+                              (float)eps, stream());
+  return out;
+}
+
 Tensor bm_residual_add_scaled(Tensor& x, const Tensor& y1, const c10::optional<Tensor>& s1,
                               const c10::optional<Tensor>& y2, const c10::optional<Tensor>& y3,
                               const c10::optional<Tensor>& s2, bool act_f32) {
@@ -390,6 +409,7 @@ Tensor bm_moe_experts(const Tensor& h, const Tensor& idx, const Tensor& wts, con
 TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("bm_rms_norm_rows(Tensor x, Tensor w, float eps, bool act_f32) -> (Tensor, Tensor)");
   m.def("bm_add_rms_norm(Tensor(a!) x, Tensor y, Tensor w, float eps, bool act_f32) -> Tensor");
+  m.def("bm_add_rms_norm_rows(Tensor(a!) x, Tensor? y, Tensor w, float eps, bool act_f32) -> Tensor");
   m.def("bm_residual_add_scaled(Tensor(a!) x, Tensor y1, Tensor? s1, Tensor? y2, Tensor? y3, Tensor? s2, "
         "bool act_f32) -> Tensor");
   m.def("bm_canon_conv(Tensor h, Tensor w, Tensor(a!) state, Tensor cu, Tensor seq_of, Tensor slots, Tensor pos, "
@@ -422,6 +442,7 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CompositeExplicitAutograd, m) {
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("bm_rms_norm_rows", &bm_rms_norm_rows);
   m.impl("bm_add_rms_norm", &bm_add_rms_norm);
+  m.impl("bm_add_rms_norm_rows", &bm_add_rms_norm_rows);
   m.impl("bm_residual_add_scaled", &bm_residual_add_scaled);
   m.impl("bm_canon_conv", &bm_canon_conv);
   m.impl("bm_norm_canon", &bm_norm_canon);

@@ -6,6 +6,8 @@
 #include <c10/core/DeviceGuard.h>
 #include <torch/library.h>
 
+#include <algorithm>
+
 #include "../hip/seqmix.h"
 
 using at::Tensor;
@@ -116,10 +118,11 @@ int64_t sm_latent_attention_fits(bool bf16, int64_t H, int64_t r, int64_t dr) {
 
 Tensor sm_latent_attention(const Tensor& q_lat, const Tensor& q_rot, const Tensor& rows, const Tensor& block_tables,
                            const Tensor& seq_of, const Tensor& pos, double scale, const c10::optional<Tensor>& gate,
-                           int64_t max_ctx, bool act_f32) {
+                           int64_t max_ctx, bool act_f32, int64_t window) {
   c10::DeviceGuard g(q_lat.device());
   TORCH_CHECK(q_lat.is_cuda() && q_lat.dim() == 3 && is_act(q_lat) && q_lat.is_contiguous(),
               "sm_latent_attention: q_lat [T, H, r] contiguous");
+  TORCH_CHECK(window >= 0 && window < (int64_t)1 << 30, "sm_latent_attention: window >= 0");
   TORCH_CHECK(act_f32 == (q_lat.scalar_type() == at::kFloat), "sm_latent_attention: activation dtype mismatch");
   const int64_t T = q_lat.size(0), H = q_lat.size(1), r = q_lat.size(2);
   TORCH_CHECK(q_rot.is_cuda() && q_rot.dim() == 3 && q_rot.scalar_type() == q_lat.scalar_type() && q_rot.size(0) == T &&
@@ -151,24 +154,28 @@ Tensor sm_latent_attention(const Tensor& q_lat, const Tensor& q_rot, const Tenso
               "sm_latent_attention: a key tile of r + dr = ", r + dr, " does not fit in LDS");
   Tensor out = at::empty({T, H, r}, q_lat.options());
   if (T == 0) return out;
-  const int nsplit = illm::sm::latent_attention_splits(bf(q_lat), (int)T, (int)H, (int)r, (int)dr, (int)max_ctx);
+  // a window spans at most window keys plus the rest of its first tile
+  const int64_t span = window > 0 ? std::min<int64_t>(max_ctx, window + 64) : max_ctx;
+  const int nsplit = illm::sm::latent_attention_splits(bf(q_lat), (int)T, (int)H, (int)r, (int)dr, (int)span);
   Tensor part;
   if (nsplit > 1) part = at::empty({T, H, nsplit, r + 2}, q_lat.options().dtype(at::kFloat));
   illm::sm::latent_attention(bf(q_lat), q_lat.data_ptr(), q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1),
                              rows.data_ptr(), (int)rows.size(1), block_tables.data_ptr<int32_t>(),
                              (int)block_tables.size(1), seq_of.data_ptr<int32_t>(), pos.data_ptr<int64_t>(), (float)scale,
                              gp, gst, out.data_ptr(), nsplit > 1 ? part.data_ptr<float>() : nullptr, nsplit, (int)T,
-                             (int)H, (int)r, (int)dr, stream());
+                             (int)H, (int)r, (int)dr, (int)window, stream());
   return out;
 }
 
 // scores f32 [R, L] (R = tokens x H rows) -> causal softmax weights; bf16 pair (hi, lo) or in place (f32)
-std::tuple<Tensor, Tensor> sm_causal_softmax(Tensor& scores, const Tensor& pos, int64_t H, double scale, bool act_f32) {
+std::tuple<Tensor, Tensor> sm_causal_softmax(Tensor& scores, const Tensor& pos, int64_t H, double scale, bool act_f32,
+                                             int64_t key0, int64_t window) {
   c10::DeviceGuard g(scores.device());
   TORCH_CHECK(scores.is_cuda() && scores.dim() == 2 && scores.scalar_type() == at::kFloat && scores.is_contiguous(),
               "sm_causal_softmax: scores f32 [R, L] contiguous");
   const int64_t R = scores.size(0), L = scores.size(1);
   TORCH_CHECK(H >= 1 && R % H == 0, "sm_causal_softmax: rows must be tokens x heads");
+  TORCH_CHECK(key0 >= 0 && window >= 0 && window < (int64_t)1 << 30, "sm_causal_softmax: key0 >= 0, window >= 0");
   check_idx(pos, at::kLong, R / H, "sm_causal_softmax: pos int64 [R / H]");
   Tensor hi, lo;
   if (!act_f32) {
@@ -176,7 +183,8 @@ std::tuple<Tensor, Tensor> sm_causal_softmax(Tensor& scores, const Tensor& pos, 
     lo = at::empty({R, L}, scores.options().dtype(at::kBFloat16));
   }
   illm::sm::causal_softmax(!act_f32, scores.data_ptr<float>(), L, pos.data_ptr<int64_t>(), (int)H, (float)scale, R, (int)L,
-                           act_f32 ? nullptr : hi.data_ptr(), act_f32 ? nullptr : lo.data_ptr(), stream());
+                           act_f32 ? nullptr : hi.data_ptr(), act_f32 ? nullptr : lo.data_ptr(), key0, (int)window,
+                           stream());
   if (act_f32) return {scores, scores};
   return {hi, lo};
 }
@@ -247,6 +255,17 @@ Tensor sm_glu_gelu(const Tensor& gu) {
   return out;
 }
 
+Tensor sm_glu_act(const Tensor& gu, int64_t act) {
+  c10::DeviceGuard g(gu.device());
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && is_act(gu) && gu.is_contiguous() && gu.size(1) % 2 == 0,
+              "sm_glu_act: [T, 2 I] contiguous bf16 / f32");
+  TORCH_CHECK(act >= 0 && act <= 2, "sm_glu_act: act 0 (tanh-GELU), 1 (ReLU) or 2 (SiLU)");
+  const int64_t T = gu.size(0), I = gu.size(1) / 2;
+  Tensor out = at::empty({T, I}, gu.options());
+  illm::sm::glu_act(bf(gu), gu.data_ptr(), out.data_ptr(), T, I, (int)act, stream());
+  return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
@@ -257,13 +276,15 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("sm_latent_kv_store(Tensor dkv, Tensor norm_w, float eps, int rank, Tensor table, Tensor pos, Tensor slots, "
         "Tensor(a!) rows) -> ()");
   m.def("sm_latent_attention(Tensor q_lat, Tensor q_rot, Tensor rows, Tensor block_tables, Tensor seq_of, Tensor pos, "
-        "float scale, Tensor? gate, int max_ctx, bool act_f32) -> Tensor");
+        "float scale, Tensor? gate, int max_ctx, bool act_f32, int window=0) -> Tensor");
   m.def("sm_latent_attention_fits(bool bf16, int H, int r, int dr) -> int");
   m.def("sm_mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, float cap, "
         "Tensor(a!) S, Tensor(b!) n, Tensor(c!) m, Tensor cu, Tensor slots, Tensor pos, int max_q) -> Tensor");
-  m.def("sm_causal_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, bool act_f32) -> (Tensor, Tensor)");
+  m.def("sm_causal_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, bool act_f32, int key0=0, int window=0) "
+        "-> (Tensor, Tensor)");
   m.def("sm_head_rms_gate(Tensor h, Tensor norm_w, Tensor gate, float eps, bool act_f32) -> Tensor");
   m.def("sm_glu_gelu(Tensor gu) -> Tensor");
+  m.def("sm_glu_act(Tensor gu, int act) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CompositeExplicitAutograd, m) {
@@ -281,4 +302,5 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("sm_causal_softmax", &sm_causal_softmax);
   m.impl("sm_head_rms_gate", &sm_head_rms_gate);
   m.impl("sm_glu_gelu", &sm_glu_gelu);
+  m.impl("sm_glu_act", &sm_glu_act);
 }

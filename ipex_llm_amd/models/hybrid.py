@@ -28,8 +28,23 @@ Building blocks (each usable by any design that lists it in its layer specs):
 * ``TokenSide``         a per-layer token input: a slice of a second
   embedding table, gated by the residual stream, projected, RMS-normed and
   added.
+* ``SSMMixer``          state-space mixer (Mamba-2 form): one input
+  projection ``[z | x | B | C | dt]``, a short causal convolution with SiLU
+  over ``[x | B | C]`` (its last inputs are state), the selective scan
+  S' = exp(-exp(A) dt) S + dt B x^T, y = S'^T C + D x over f32 state slots,
+  then y silu(z), a group RMS norm and the output projection.
+* ``MaskedAttention``   grouped-query attention over paged ``[keys | values]``
+  rows with separate value size, optional projection biases, RMS norm of
+  queries and keys per head or over the whole projection, rotary positions in
+  either pair layout, a causal / sliding-window / chunked view of the past,
+  an optional per-head sink in the softmax, and optionally the keys and
+  values of an earlier layer (``kv_from``) instead of its own.
+* ``LatentAttention`` also takes a sliding window, the half-split rotary layout
+  (folded into the weights' row order) and an element-wise output gate.
 
-Block layouts.  ``post_norm`` (``HybridLayer``): the sublayers read the
+Block layouts.  ``pre_norm`` (``PreNormLayer``): x += mixer(norm1(x)),
+x += ff(norm2(x)) with vector RMS norms; each sublayer's result is added by
+the launch that also forms the next norm.  ``post_norm`` (``HybridLayer``): the sublayers read the
 residual stream ``x`` itself and their *output* is normalised:
 x += mult * LN(mixer(x)), x += mult * LN(ff(x)).  ``parallel``
 (``ParallelLayer``): one norm, both sublayers read it, their scaled results
@@ -54,7 +69,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ..ops import blockmix as BM
+from ..ops import maskattn as MA
 from ..ops import seqmix as SM
+from ..ops import ssm as SSM
 from .decoder import AttnMeta
 
 
@@ -64,6 +81,13 @@ class RotarySpec:
     dims: int
     base: float = 10000.0
     scaling: Optional[dict] = None          # YaRN: factor, original, fast, slow
+    layout: Optional[str] = None            # "pairs" (2i, 2i+1) | "half" (i, i + dims/2); None: the mixer's own
+
+
+@dataclass
+class MaskSpec:
+    kind: str = "causal"                    # "causal" | "window" (itself and size - 1 before) | "chunk" (aligned blocks)
+    size: int = 0
 
 
 @dataclass
@@ -76,6 +100,33 @@ class LatentAttentionSpec:
     scale: float
     rot: RotarySpec = None
     out_gate: bool = True
+    gate: str = "head"                      # "head": one gate per head | "element": one per value of the joined heads
+    window: int = 0                         # > 0: a token sees itself and the window - 1 tokens before it
+
+
+@dataclass
+class SSMSpec:
+    heads: int
+    vdim: int                               # values per head (inner = heads * vdim)
+    state: int                              # N
+    groups: int                             # B / C groups; head h reads group h // (heads / groups)
+    taps: int                               # of the convolution over [x | B | C]
+    norm_groups: int = 1
+
+
+@dataclass
+class MaskedAttentionSpec:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: Optional[RotarySpec] = None        # on the first rot.dims values of every head
+    mask: MaskSpec = None
+    qk_norm: str = "whole"                  # "none" | "head" (weights [dim]) | "whole" (weights [heads dim])
+    bias: bool = True                       # q / k / v projections carry biases
+    sink: bool = True                       # a learned number per head in the softmax's denominator
+    kv_from: Optional[int] = None           # read this layer's cache rows instead of projecting keys and values
 
 
 @dataclass
@@ -89,6 +140,7 @@ class MLSTMSpec:
 @dataclass
 class DenseFFSpec:
     ff: int
+    act: str = "gelu_tanh"                  # "gelu_tanh" | "relu" | "silu" on the gate rows
 
 
 @dataclass
@@ -147,7 +199,8 @@ class HybridSpec:
     residual_mult: float = 1.0
     bigram: Optional[BigramSpec] = None
     final_softcap: float = 0.0              # read by the engines' shared helpers
-    block: str = "post_norm"                # "post_norm" | "parallel"
+    logit_scale: float = 1.0                # the logits are multiplied by it
+    block: str = "post_norm"                # "post_norm" | "parallel" | "pre_norm"
     norm: str = "layer_norm"                # "layer_norm" | "rms_scalar" (one number) | "rms" (a vector)
     layer_scale: bool = False               # parallel blocks: per-coordinate scales on both sublayers' results
     canon_taps: int = 0                     # parallel blocks: taps of the convolution in front of the mixer (0: none)
@@ -166,6 +219,17 @@ class LatentAttention(nn.Module):
         super().__init__()
         self.s = s
         H, r = s.heads, s.kv_rank
+        if s.rot is not None and s.rot.layout == "half":
+            # half-split pairs (i, i + dims / 2) -> the kernels' neighbouring pairs (2 i, 2 i + 1): the same
+            # reordering of the rotated rows of W_q (every head) and of W_dkv leaves every score unchanged
+            n = s.rot.dims
+            perm = torch.arange(s.rot_dim)
+            perm[:n] = torch.stack([torch.arange(n // 2), torch.arange(n // 2) + n // 2], 1).reshape(-1)
+            w_q = w_q.view(H, s.dim + s.rot_dim, -1)
+            w_q = torch.cat([w_q[:, :s.dim], w_q[:, s.dim:][:, perm.to(w_q.device)]], 1).reshape(H * (s.dim + s.rot_dim), -1)
+            w_dkv = torch.cat([w_dkv[:r], w_dkv[r:][perm.to(w_dkv.device)]], 0)
+        if s.out_gate and s.gate not in ("head", "element"):
+            raise ValueError(f"unknown gate kind {s.gate!r}")
         # one projection launch: [q | dkv | gate] rows
         parts = [w_q, w_dkv] + ([w_g] if w_g is not None else [])
         self.w_in = nn.Parameter(torch.cat(parts, 0).contiguous(), requires_grad=False)
@@ -192,15 +256,19 @@ class LatentAttention(nn.Module):
         q = y[:, :self.n_q].reshape(T, H, s.dim + s.rot_dim).contiguous()
         dkv = y[:, self.n_q:self.n_q + self.n_dkv]
         gate = y[:, self.n_q + self.n_dkv:] if s.out_gate else None
+        head_gate = gate if s.gate == "head" else None
         table = self.table
         SM.latent_kv_store(dkv, self.dkv_norm, eps, s.kv_rank, table, pos, slots, cache.rows[li])
         SM.rope_rows_(q, s.dim, table, pos)
         # absorbed up-projection of the keys: per-head [T, dim] x [dim, r]
         q_lat = torch.bmm(q[..., :s.dim].transpose(0, 1), self.w_uk).transpose(0, 1)
         o_lat = SM.latent_attention(q_lat, q[..., s.dim:], cache.rows[li], meta.block_tables, meta.seq_of, pos,
-                                    s.scale, gate, meta.q_lens_host, meta.seq_lens_host, xa.dtype)
+                                    s.scale, head_gate, meta.q_lens_host, meta.seq_lens_host, xa.dtype,
+                                    window=s.window)
         o = torch.bmm(o_lat.transpose(0, 1), self.w_uv_t).transpose(0, 1).reshape(T, H * s.vdim)
-        return F.linear(o, self.w_o)
+        if gate is not None and s.gate == "element":
+            o = MA.sigmoid_gate(o, gate)
+        return BM.linear(o, self.w_o)
 
 
 class MLSTM(nn.Module):
@@ -238,13 +306,127 @@ class MLSTM(nn.Module):
 
 
 class DenseFF(nn.Module):
-    def __init__(self, w_gate, w_up, w_down):
+    """``W_down (act(W_gate h) * (W_up h))``"""
+
+    def __init__(self, w_gate, w_up, w_down, act: str = "gelu_tanh"):
         super().__init__()
+        if act not in SM.GLU_ACTS:
+            raise ValueError(f"unknown feed-forward activation {act!r}")
+        self.act = act
         self.w_gu = nn.Parameter(torch.cat([w_gate, w_up], 0).contiguous(), requires_grad=False)
         self.w_down = nn.Parameter(w_down, requires_grad=False)
 
     def forward(self, xa):
-        return F.linear(SM.glu_gelu(F.linear(xa, self.w_gu)), self.w_down)
+        if self.act == "gelu_tanh":
+            return F.linear(SM.glu_gelu(F.linear(xa, self.w_gu)), self.w_down)
+        return BM.linear(SM.glu_act(BM.linear(xa, self.w_gu), self.act), self.w_down)
+
+
+class SSMMixer(nn.Module):
+    """``w_in`` rows ``[z (inner) | x (inner) | B (G N) | C (G N) | dt (heads)]``; ``conv_w`` [inner + 2 G N, taps]
+    (last column: the current token) with bias ``conv_b``; ``dt_bias`` / ``a_log`` / ``d_skip`` [heads]; ``norm``
+    [inner]."""
+    cache_kind = "state"
+
+    def __init__(self, s: SSMSpec, w_in, conv_w, conv_b, dt_bias, a_log, d_skip, norm, w_o):
+        super().__init__()
+        if s.heads % s.groups:
+            raise ValueError("heads must be a multiple of groups")
+        if (s.heads * s.vdim) % s.norm_groups:
+            raise ValueError("heads * vdim must split into norm_groups equal parts")
+        if s.taps < 1 or s.taps > 16:
+            raise ValueError("1 <= conv taps <= 16")
+        if s.state > SSM.SCAN_MAX_STATE:
+            raise ValueError(f"state size above {SSM.SCAN_MAX_STATE}")
+        self.s = s
+        self.inner, self.chan = s.heads * s.vdim, s.heads * s.vdim + 2 * s.groups * s.state
+        self.w_in = nn.Parameter(w_in, requires_grad=False)
+        self.conv_w = nn.Parameter(conv_w.float().contiguous(), requires_grad=False)
+        self.conv_b = nn.Parameter(conv_b.float().contiguous(), requires_grad=False)
+        self.dt_bias = nn.Parameter(dt_bias.float().contiguous(), requires_grad=False)
+        self.a_log = nn.Parameter(a_log.float().contiguous(), requires_grad=False)
+        self.d_skip = nn.Parameter(d_skip.float().contiguous(), requires_grad=False)
+        self.norm = nn.Parameter(norm, requires_grad=False)
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+
+    def cache_spec(self):
+        s = self.s
+        return ("state", {"S": (s.heads, s.state, s.vdim), "conv": (s.taps - 1, self.chan)})
+
+    def ensure_table(self, max_pos: int):
+        return None
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        s = self.s
+        T, H, inner, GN = xa.shape[0], s.heads, self.inner, s.groups * s.state
+        y = BM.linear(xa, self.w_in)
+        z, u, dt = y[:, :inner], y[:, inner:inner + self.chan], y[:, inner + self.chan:]
+        st = cache.state[li]
+        xbc = SSM.conv_silu(u, self.conv_w, self.conv_b, st["conv"], meta.cu_q, meta.seq_of, meta.state_slots, pos,
+                            meta.q_lens_host)
+        yy = SSM.selective_scan(xbc[:, :inner].view(T, H, s.vdim), xbc[:, inner:inner + GN].view(T, s.groups, s.state),
+                                xbc[:, inner + GN:].view(T, s.groups, s.state), dt, self.dt_bias, self.a_log,
+                                self.d_skip, st["S"], meta.cu_q, meta.state_slots, pos, meta.q_lens_host)
+        o = SSM.gated_group_norm(yy.view(T, inner), z, self.norm, s.norm_groups, eps, xa.dtype)
+        return BM.linear(o, self.w_o)
+
+
+class MaskedAttention(nn.Module):
+    """``w_q`` [H d, W], ``w_k`` [G d, W], ``w_v`` [G dv, W] (``w_k`` / ``w_v`` None with ``kv_from``), biases or
+    None, norm weights per ``qk_norm``, ``sink`` [H] or None, ``w_o`` [W, H dv]."""
+    cache_kind = "rows"
+
+    def __init__(self, s: MaskedAttentionSpec, w_q, w_k, w_v, b_q, b_k, b_v, q_norm, k_norm, sink, w_o):
+        super().__init__()
+        if s.heads % s.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if s.mask is None or s.mask.kind not in MA.MASKS or (s.mask.kind != "causal" and s.mask.size < 1):
+            raise ValueError("mask: causal, or window / chunk with a size of at least 1")
+        if s.qk_norm not in ("none", "head", "whole"):
+            raise ValueError(f"unknown qk_norm {s.qk_norm!r}")
+        self.s = s
+        shared = s.kv_from is not None
+        self.w_in = nn.Parameter((w_q if shared else torch.cat([w_q, w_k, w_v], 0)).contiguous(), requires_grad=False)
+        self.b_in = None
+        if s.bias:
+            self.b_in = nn.Parameter((b_q if shared else torch.cat([b_q, b_k, b_v], 0)).contiguous(), requires_grad=False)
+        self.q_norm = nn.Parameter(q_norm, requires_grad=False) if q_norm is not None else None
+        self.k_norm = nn.Parameter(k_norm, requires_grad=False) if k_norm is not None else None
+        self.sink = nn.Parameter(sink.float().contiguous(), requires_grad=False) if sink is not None else None
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+        self.table: Optional[torch.Tensor] = None
+
+    def cache_spec(self):
+        s = self.s
+        return None if s.kv_from is not None else ("rows", s.kv_heads * (s.dim + s.vdim))
+
+    def ensure_table(self, max_pos: int):
+        if self.s.rot is None or self.s.rot.dims == 0:
+            return None
+        if self.table is None or self.table.shape[0] < max_pos or self.table.device != self.w_o.device:
+            n = max(256, 1 << (max_pos - 1).bit_length())
+            self.table = SM.rope_table(n, self.s.rot.dims, self.s.rot.base, self.s.rot.scaling).to(self.w_o.device)
+        return self.table
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        s = self.s
+        T, H, G, d, dv = xa.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        y = BM.linear(xa, self.w_in, self.b_in)
+        q = y[:, :H * d].view(T, H, d)
+        layout = (s.rot.layout if s.rot is not None else None) or "half"
+        if s.kv_from is None:
+            k = y[:, H * d:(H + G) * d].view(T, G, d)
+            v = y[:, (H + G) * d:].view(T, G, dv)
+            rows = cache.rows[li]
+            qf = MA.qkv_norm_rope_store(q, k, v, self.q_norm, self.k_norm, s.qk_norm == "whole", eps, self.table,
+                                        layout, pos, slots, rows)
+        else:
+            rows = cache.rows[s.kv_from]
+            qf = MA.qkv_norm_rope_store(q, None, None, self.q_norm, None, s.qk_norm == "whole", eps, self.table,
+                                        layout, pos, slots, None)
+        o = MA.masked_attention(qf, rows, G, dv, meta.block_tables, meta.seq_of, pos, s.scale, s.mask.kind, s.mask.size,
+                                self.sink, meta.q_lens_host, meta.seq_lens_host, xa.dtype)
+        return BM.linear(o, self.w_o)
 
 
 class GroupedAttention(nn.Module):
@@ -356,6 +538,30 @@ class HybridLayer(nn.Module):
         return xa
 
 
+class PreNormLayer(nn.Module):
+    """x += mixer(norm1(x)); x += ff(norm2(x)).  ``carry`` is the previous sublayer's result that is not yet in
+    ``x`` (None at the first layer): the launch that forms a norm adds it first, and the layer hands its own last
+    result on the same way (the model adds the final one with its own norm)."""
+
+    def __init__(self, mixer: nn.Module, norm1: torch.Tensor, mlp: Optional[nn.Module], norm2: Optional[torch.Tensor]):
+        super().__init__()
+        self.mixer, self.mlp = mixer, mlp
+        self.norm1 = nn.Parameter(norm1, requires_grad=False)
+        self.norm2 = nn.Parameter(norm2, requires_grad=False) if norm2 is not None else None
+
+    def cache_specs(self):
+        return [self.mixer.cache_spec()]
+
+    def forward(self, x, carry, ids, pos, slots, meta, cache, li: int, model):
+        s, act = model.spec, model.dtype
+        h = BM.add_rms_norm_rows_(x, carry, self.norm1, s.norm_eps, act)
+        y = self.mixer(h, pos, slots, meta, cache, li, s.norm_eps)
+        if self.mlp is None:
+            return y
+        h = BM.add_rms_norm_rows_(x, y, self.norm2, s.norm_eps, act)
+        return self.mlp(h)
+
+
 class ParallelLayer(nn.Module):
     """h = norm(x);  x += ls1 * mixer(h + conv(h)) + ls2 * ff(h);  then the
     token-side input.  ``canon`` [W, taps] or None, ``ls1`` / ``ls2`` [W] or
@@ -395,7 +601,8 @@ class ParallelLayer(nn.Module):
 # name -> (spec class, module class): a design's config reader maps its layer
 # types onto these
 MIXERS: Dict[str, tuple] = {"latent_attention": (LatentAttentionSpec, LatentAttention), "mlstm": (MLSTMSpec, MLSTM),
-                            "grouped_attention": (GroupedAttentionSpec, GroupedAttention)}
+                            "grouped_attention": (GroupedAttentionSpec, GroupedAttention),
+                            "ssm": (SSMSpec, SSMMixer), "masked_attention": (MaskedAttentionSpec, MaskedAttention)}
 
 
 # ---------------------------------------------------------------------- model
@@ -424,7 +631,7 @@ class HybridCausalLM(nn.Module):
 
     @property
     def has_state(self) -> bool:
-        return any(c[0] == "state" for L in self.layers for c in L.cache_specs())
+        return any(c is not None and c[0] == "state" for L in self.layers for c in L.cache_specs())
 
     def graph_max_batch(self) -> int:
         return 0                    # ragged steps are launched eagerly
@@ -435,7 +642,7 @@ class HybridCausalLM(nn.Module):
 
     def cache_bytes_per_token(self) -> int:
         eb = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(c[1] * eb for L in self.layers for c in L.cache_specs() if c[0] == "rows")
+        return sum(c[1] * eb for L in self.layers for c in L.cache_specs() if c is not None and c[0] == "rows")
 
     def make_cache(self, max_tokens: int, batch: int = 1, block_size: int = 64, kv_fp8: int = 0,
                    num_blocks: Optional[int] = None, num_slots: Optional[int] = None):
@@ -482,19 +689,24 @@ class HybridCausalLM(nn.Module):
             x = SM.embed_bigram(ids, meta.prev_ids, self.embed_tokens, self.bigram, b.mul_prev, b.mul_cur)
         else:
             x = F.embedding(ids, self.embed_tokens).float()
-        xa = x if act == torch.float32 else x.to(act)
+        pre = s.block == "pre_norm"         # ``xa`` is then the last sublayer's result, still to be added to x
+        xa = None if pre else (x if act == torch.float32 else x.to(act))
         for li, L in enumerate(self.layers):
             xa = L(x, xa, ids, pos, slots, meta, cache, li, self)
             if self.capture_layers is not None:
-                self.capture_layers.append(x.clone())
+                self.capture_layers.append(x + xa.float() if pre else x.clone())
         if not self.last_stage:
-            return x
+            return x.add_(xa.float()) if pre and xa is not None else x
         if logits_idx is not None:
             x = x.index_select(0, logits_idx)
-        if s.norm == "layer_norm":
+            xa = xa.index_select(0, logits_idx) if pre and xa is not None else xa
+        if pre:
+            xn = BM.add_rms_norm_rows_(x, xa, self.norm, s.norm_eps, act)
+        elif s.norm == "layer_norm":
             xn = SM.layer_norm_f32(x, self.norm, s.norm_eps, act)
         else:
             xn = BM.rms_norm_rows(x, self.norm, s.norm_eps, act)[1]
         if return_hidden:
             return xn
-        return BM.linear(xn, self.lm_head).float()
+        logits = BM.linear(xn, self.lm_head).float()
+        return logits.mul_(s.logit_scale) if s.logit_scale != 1.0 else logits

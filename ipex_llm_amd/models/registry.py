@@ -18,6 +18,7 @@ import torch
 NATIVE_ARCHITECTURES = {
     "Zamelix": "ipex_llm_amd.models.zamelix",
     "Masezen": "ipex_llm_amd.models.masezen",
+    "Vogolix": "ipex_llm_amd.models.vogolix",
 }
 
 

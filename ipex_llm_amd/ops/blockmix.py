@@ -23,7 +23,7 @@ import torch.nn.functional as F
 
 from .seqmix import native, _mm_f32
 
-__all__ = ["linear", "rms_norm_rows", "canon_conv", "norm_canon", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
+__all__ = ["linear", "rms_norm_rows", "add_rms_norm_rows_", "canon_conv", "norm_canon", "qk_norm_rope_store", "talk_attention", "relu_sq", "glu_clamp",
            "residual_add_scaled_", "side_gate", "add_rms_norm_", "moe_route", "moe_experts"]
 
 
@@ -32,14 +32,14 @@ def _ops():
 
 
 # ------------------------------------------------------------------ projections
-def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """``x W^T`` for rows ``x`` [T, K] and ``w`` [N, K]: decode-size steps (at most 16 rows, 16-bit) stream the
-    weight once through the skinny-GEMM kernel the dense decoders use (csrc/hip/dense_gemv.hip), everything
+def linear(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x W^T (+ b)`` for rows ``x`` [T, K] and ``w`` [N, K]: decode-size steps (at most 16 rows, 16-bit) stream
+    the weight once through the skinny-GEMM kernel the dense decoders use (csrc/hip/dense_gemv.hip), everything
     else is a library GEMM."""
     if x.is_cuda and x.dim() == 2 and x.shape[0] <= 16 and x.dtype == torch.bfloat16 and w.dtype == x.dtype and \
             x.shape[1] % 8 == 0 and w.is_contiguous() and native(x):
-        return _ops().dense_linear(x, w, None)
-    return F.linear(x, w)
+        return _ops().dense_linear(x, w, b)
+    return F.linear(x, w, b)
 
 
 # ------------------------------------------------------------------ norms
@@ -62,6 +62,19 @@ def add_rms_norm_(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, eps: float,
     yf = y.float()
     x.add_(yf * torch.rsqrt((yf * yf).mean(-1, keepdim=True) + eps) * w.float())
     return x if act_dtype == torch.float32 else x.to(act_dtype)
+
+
+def add_rms_norm_rows_(x: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor, eps: float,
+                       act_dtype: torch.dtype) -> torch.Tensor:
+    """``x += y`` on the f32 residual rows in place (``y`` in the activation
+    dtype, or None for nothing to add), then ``x / sqrt(mean(x^2) + eps) * w``
+    (``w`` [W]) in ``act_dtype``: the residual sum of one sublayer and the norm
+    in front of the next in one pass."""
+    if native(x):
+        return _ops().bm_add_rms_norm_rows(x, None if y is None else y.contiguous(), w, eps, act_dtype == torch.float32)
+    if y is not None:
+        x.add_(y.float())
+    return (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.float()).to(act_dtype)
 
 
 def residual_add_scaled_(x: torch.Tensor, y1: torch.Tensor, s1: Optional[torch.Tensor], y2: Optional[torch.Tensor],

@@ -1,0 +1,250 @@
+"""Grouped-query attention over paged ``[keys | values]`` rows with a bounded
+view of the past (a sliding window or position-aligned chunks) and an optional
+sink in the softmax, plus the fused step in front of it: RMS norm of queries
+and keys (per head or over the whole projection), rotary positions in either
+pair layout, and the cache append.  Used by ``models/hybrid.py``
+``MaskedAttention``.
+
+Every op takes a *ragged step* like ``ops/seqmix.py``.  GPU tensors run the
+HIP kernels of ``csrc/hip/maskattn.hip``; CPU tensors run the torch forms
+below, which are also what the kernels are tested against.
+
+Precision (both paths): norms, angles, scores, the softmax with its sink and
+the weighted sum are f32 whatever the activation dtype is; the queries leave
+the first step as f32 and are never rounded.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional
+
+import torch
+
+from .seqmix import native, _mm_f32
+
+__all__ = ["MASKS", "LAYOUTS", "first_visible", "qkv_norm_rope_store", "masked_attention", "sigmoid_gate"]
+
+MASKS = {"causal": 0, "window": 1, "chunk": 2}
+LAYOUTS = {"pairs": 0, "half": 1}
+
+
+def _ops():
+    return torch.ops.ipex_llm_amd
+
+
+def first_visible(pos: torch.Tensor, mask: str, size: int) -> torch.Tensor:
+    """the first key position a query at ``pos`` sees: 0 (causal), pos - size + 1
+    clamped at 0 (window: itself and the size - 1 tokens before it), or the start
+    of pos's chunk (chunks of ``size`` positions counted from position 0)"""
+    if mask == "causal":
+        return torch.zeros_like(pos)
+    if mask == "window":
+        return (pos - (size - 1)).clamp(min=0)
+    if mask == "chunk":
+        return pos - pos % size
+    raise ValueError(f"unknown mask {mask!r}")
+
+
+def _turn(x: torch.Tensor, cs: torch.Tensor, layout: str) -> torch.Tensor:
+    """rotate the first ``2 * cs.shape[-2]`` values of every head of x f32 [T, heads, n]; cs [T, 1, dims / 2, 2]"""
+    dims = 2 * cs.shape[-2]
+    c, s = cs[..., 0], cs[..., 1]
+    out = x.clone()
+    if layout == "half":
+        u, v = x[..., :dims // 2], x[..., dims // 2:dims]
+        out[..., :dims // 2] = u * c - v * s
+        out[..., dims // 2:dims] = v * c + u * s
+    else:
+        u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+        out[..., 0:dims:2] = u * c - v * s
+        out[..., 1:dims:2] = v * c + u * s
+    return out
+
+
+def qkv_norm_rope_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                        q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], whole: bool, eps: float,
+                        table: Optional[torch.Tensor], layout: str, pos: torch.Tensor, slots: torch.Tensor,
+                        rows: Optional[torch.Tensor]) -> torch.Tensor:
+    """RMS norm and rotary positions of ``q`` [T, H, d] and ``k`` [T, G, d]
+    (strided views allowed), and one cache row per token.
+
+    ``whole``: the norm runs over all heads of a token at once (weights of the
+    whole projection's size, [H d] and [G d]); otherwise per head (weights [d],
+    shared by the heads).  A missing weight means no norm.  The rotation turns
+    the first ``2 * table.shape[1]`` values of every head, pairing value i with
+    i + dims / 2 (``layout`` "half") or 2 i with 2 i + 1 ("pairs"); no table: no
+    rotation.  When ``k`` is given, ``[keys (normed, rotated) | v as projected]``
+    is written at row index ``slots`` of the paged pool ``rows``
+    [blocks, bs, G d + G dv]; a layer that reads another layer's rows passes
+    ``k = v = rows = None``.  Returns the queries f32 [T, H, d]."""
+    T, H, d = q.shape
+    if native(q):
+        return _ops().ma_qkv_norm_rope_store(q, k, v, q_norm, k_norm, whole, eps, table, LAYOUTS[layout], pos, slots,
+                                             rows)
+    cs = table[pos.long()][:, None] if table is not None else None
+
+    def prep(x, w):
+        x = x.float()
+        if w is not None:
+            if whole:
+                n = x.shape[1] * x.shape[2]
+                flat = x.reshape(T, n)
+                x = (flat * torch.rsqrt((flat * flat).mean(-1, keepdim=True) + eps) * w.float()).view(x.shape)
+            else:
+                x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.float()
+        return _turn(x, cs, layout) if cs is not None else x
+
+    qf = prep(q, q_norm)
+    if k is not None:
+        kf = prep(k, k_norm)
+        flat = rows.view(-1, rows.shape[-1])
+        flat.index_copy_(0, slots.long(), torch.cat([kf.reshape(T, -1), v.float().reshape(T, -1)], -1).to(rows.dtype))
+    return qf.contiguous()
+
+
+# GPU paths by portion: decoded tokens and short or unaligned pieces run the one-pass kernel, a workgroup per
+# (token, key head).  With chunks, a portion's whole chunks (from a chunk's first position to its last) see only
+# their own keys: at least GEMM_MIN_CHUNK tokens per chunk and they run as batched library products over the
+# chunks, with the fused softmax (sink, causal mask inside the chunk) between them.
+GEMM_MIN_CHUNK = int(os.environ.get("ILLM_MASKATTN_GEMM_MIN", "128"))
+
+
+def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block_tables: torch.Tensor,
+                     seq_of: torch.Tensor, pos: torch.Tensor, scale: float, mask: str, size: int,
+                     sink: Optional[torch.Tensor], q_lens: List[int], ctx_lens: List[int],
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """Grouped-query attention over paged rows ``[keys (G d) | values (G dv)]``.
+    For token t (position p), query head h (key / value head h // (H / G)) and
+    the visible keys ``first_visible(p) <= j <= p``:
+
+        s_j = (q[t, h] . key_j) * scale
+        w_j = exp(s_j) / (sum_visible exp(s_i) + exp(sink[h]))      (no sink: the plain softmax)
+        out[t, h] = sum_j w_j value_j
+
+    The sink is one more term of the denominator: it has no key and no value,
+    is not scaled and counts once.  ``q`` f32 [T, H, d]; everything is f32.
+    Returns [T, H dv] in ``out_dtype``."""
+    T, H, d = q.shape
+    if native(q):
+        return _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, float(scale), mask, int(size), sink,
+                                     q_lens, ctx_lens, out_dtype)
+    rep = H // G
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    bs = rows.shape[1]
+    t0 = 0
+    for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
+        if n == 0:
+            continue
+        nb = (L + bs - 1) // bs
+        kv = rows[block_tables[b, :nb].long()].reshape(nb * bs, -1)[:L].float()
+        kk = kv[:, :G * d].view(L, G, d).repeat_interleave(rep, 1)
+        vv = kv[:, G * d:].view(L, G, dv).repeat_interleave(rep, 1)
+        p = pos[t0:t0 + n].long()
+        sc = torch.einsum("thd,lhd->htl", q[t0:t0 + n], kk) * scale
+        j = torch.arange(L, device=sc.device)[None, :]
+        vis = (j <= p[:, None]) & (j >= first_visible(p, mask, size)[:, None])
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        top = sc.max(-1, keepdim=True).values
+        if sink is not None:
+            top = torch.maximum(top, sink.float()[:, None, None])
+        e = torch.exp(sc - top)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sink.float()[:, None, None] - top)
+        out[t0:t0 + n] = torch.einsum("htl,lhd->thd", e / den, vv)
+        t0 += n
+    return out.reshape(T, H * dv).to(out_dtype)
+
+
+def _chunk_blocks_gemm(q, rows, table_row, G, dv, scale, size, sink, t0, c0, nc, out):
+    """``nc`` whole chunks of one sequence, starting at chunk index ``c0`` with the step's token ``t0``: scores and
+    weighted sums as batched products over (chunk, key head), the sink softmax fused between them"""
+    _, H, d = q.shape
+    rep = H // G
+    bs = rows.shape[1]
+    f32 = rows.dtype == torch.float32
+    n = nc * size
+    lo = c0 * size
+    # the chunks' rows in position order (gathered through the block table)
+    p = torch.arange(lo, lo + n, device=q.device)
+    ridx = table_row.long()[p // bs] * bs + p % bs
+    kv = rows.view(-1, rows.shape[-1]).index_select(0, ridx)
+    kk = kv[:, :G * d].reshape(nc, size, G, d).permute(0, 2, 3, 1).reshape(nc * G, d, size)
+    vv = kv[:, G * d:].reshape(nc, size, G, dv).permute(0, 2, 1, 3).reshape(nc * G, size, dv)
+    qq = q[t0:t0 + n].view(nc, size, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, size * rep, d)
+    if f32:
+        sc = torch.bmm(qq, kk)
+    else:                                       # f32 queries against 16-bit keys: hi + lo halves of q
+        qh = qq.to(rows.dtype)
+        ql = (qq - qh.float()).to(rows.dtype)
+        sc = torch.bmm(qh, kk, out_dtype=torch.float32) + torch.bmm(ql, kk, out_dtype=torch.float32)
+    hi, lo_w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, f32)
+    hi = hi.view(nc * G, size * rep, size)
+    if f32:
+        o = torch.bmm(hi, vv)
+    else:
+        o = torch.bmm(hi, vv, out_dtype=torch.float32) + torch.bmm(lo_w.view_as(hi), vv, out_dtype=torch.float32)
+    o = o.view(nc, G, size, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
+    out[t0:t0 + n] = o.to(out.dtype)
+
+
+def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask, size, sink, q_lens, ctx_lens,
+                          out_dtype):
+    T, H, d = q.shape
+    f32 = out_dtype == torch.float32
+    q = q.contiguous()
+    code = MASKS[mask]
+    big = mask == "chunk" and size >= GEMM_MIN_CHUNK and max(q_lens) >= size and _bmm_f32_ok(rows.dtype)
+    if not big:
+        return _ops().ma_masked_attention(q, rows, G, dv, block_tables, seq_of, pos, scale, code, size, sink,
+                                          max(ctx_lens), f32)
+    out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+    rest, rest_ctx, t0 = [], 1, 0
+    for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
+        p0 = L - n                                                   # position of the portion's first token
+        c0 = -(-p0 // size)                                          # first chunk that starts inside the portion
+        nc = (L - c0 * size) // size if L >= c0 * size else 0
+        if nc > 0:
+            a = t0 + c0 * size - p0
+            _chunk_blocks_gemm(q, rows, block_tables[b], G, dv, scale, size, sink, a, c0, nc, out)
+            if a > t0:
+                rest.append(torch.arange(t0, a, device=q.device))
+            if a + nc * size < t0 + n:
+                rest.append(torch.arange(a + nc * size, t0 + n, device=q.device))
+            if a > t0 or a + nc * size < t0 + n:
+                rest_ctx = max(rest_ctx, L)
+        elif n:
+            rest.append(torch.arange(t0, t0 + n, device=q.device))
+            rest_ctx = max(rest_ctx, L)
+        t0 += n
+    if rest:
+        idx = torch.cat(rest)
+        out[idx] = _ops().ma_masked_attention(q[idx].contiguous(), rows, G, dv, block_tables, seq_of[idx].contiguous(),
+                                              pos[idx].contiguous(), scale, code, size, sink, rest_ctx, f32)
+    return out
+
+
+_bmm_out_f32: Optional[bool] = None
+
+
+def _bmm_f32_ok(dtype) -> bool:
+    """batched 16-bit products with f32 results (torch.bmm out_dtype)"""
+    global _bmm_out_f32
+    if dtype == torch.float32:
+        return True
+    if _bmm_out_f32 is None:
+        try:
+            a = torch.zeros(1, 16, 16, dtype=dtype, device="cuda")
+            torch.bmm(a, a, out_dtype=torch.float32)
+            _bmm_out_f32 = True
+        except (TypeError, RuntimeError):
+            _bmm_out_f32 = False
+    return _bmm_out_f32
+
+
+def sigmoid_gate(o: torch.Tensor, gate_pre: torch.Tensor) -> torch.Tensor:
+    """``o * sigmoid(gate_pre)`` element by element (f32 math), o's dtype;
+    ``gate_pre`` may be a strided view of a projection's result."""
+    if native(o):
+        return _ops().ma_sigmoid_gate(o.contiguous(), gate_pre)
+    return (o.float() * torch.sigmoid(gate_pre.float())).to(o.dtype)

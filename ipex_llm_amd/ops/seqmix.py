@@ -24,7 +24,7 @@ import torch
 import torch.nn.functional as F
 
 __all__ = ["embed_bigram", "add_scaled_layer_norm_", "layer_norm_f32", "latent_kv_store", "rope_rows_",
-           "latent_attention", "mlstm_scan", "head_rms_gate", "glu_gelu", "rope_table", "native"]
+           "latent_attention", "mlstm_scan", "head_rms_gate", "glu_gelu", "glu_act", "GLU_ACTS", "rope_table", "native"]
 
 
 def native(t: torch.Tensor) -> bool:
@@ -145,20 +145,22 @@ def latent_kv_store(dkv: torch.Tensor, norm_w: torch.Tensor, eps: float, rank: i
 # ------------------------------------------------------------------ latent attention
 def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, rows: torch.Tensor, block_tables: torch.Tensor,
                      seq_of: torch.Tensor, pos: torch.Tensor, scale: float, gate: Optional[torch.Tensor],
-                     q_lens: List[int], ctx_lens: List[int], out_dtype: torch.dtype) -> torch.Tensor:
+                     q_lens: List[int], ctx_lens: List[int], out_dtype: torch.dtype, window: int = 0) -> torch.Tensor:
     """Causal softmax attention in the latent space over the paged rows
     ``[latent (r) | rotated key (dr)]``: for token t of sequence b and head h
 
         s_j = (q_lat[t, h] . c_j + q_rot[t, h] . kr_j) * scale      for j <= pos[t]
         out[t, h] = sigmoid(gate[t, h]) * sum_j softmax(s)_j c_j     [r]
 
-    (scores, softmax and the weighted sum in f32).  ``q_rot`` may be a strided
-    view.  ``q_lens`` / ``ctx_lens``: host copies of every sequence's new-token
-    count and key count."""
+    (scores, softmax and the weighted sum in f32).  ``window`` > 0: only the
+    keys pos[t] - window < j <= pos[t] count (the token itself and the
+    window - 1 before it).  ``q_rot`` may be a strided view.  ``q_lens`` /
+    ``ctx_lens``: host copies of every sequence's new-token count and key count."""
     T, H, r = q_lat.shape
+    window = int(window or 0)
     if native(q_lat):
         return _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, float(scale), gate, q_lens,
-                                     ctx_lens, out_dtype)
+                                     ctx_lens, out_dtype, window)
     out = torch.empty(T, H, r, dtype=torch.float32, device=q_lat.device)
     bs = rows.shape[1]
     t0 = 0
@@ -170,7 +172,8 @@ def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, rows: torch.Tenso
         c, kr = kv[:, :r], kv[:, r:]
         ql, qr = q_lat[t0:t0 + n].float(), q_rot[t0:t0 + n].float()
         sc = (torch.einsum("thr,lr->thl", ql, c) + torch.einsum("thd,ld->thl", qr, kr)) * scale
-        vis = torch.arange(L, device=sc.device)[None, :] <= pos[t0:t0 + n].long()[:, None]
+        j, p = torch.arange(L, device=sc.device)[None, :], pos[t0:t0 + n].long()[:, None]
+        vis = (j <= p) & (j > p - window) if window > 0 else j <= p
         sc = sc.masked_fill(~vis[:, None, :], float("-inf"))
         out[t0:t0 + n] = torch.einsum("thl,lr->thr", torch.softmax(sc, -1), c)
         t0 += n
@@ -206,7 +209,7 @@ def _mm_f32(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return a.float() @ b.float()
 
 
-def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n: int) -> torch.Tensor:
+def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n: int, window: int = 0) -> torch.Tensor:
     """one sequence's portion of n >= GEMM_MIN_Q tokens ending at key count L -> f32 [n, H, r]"""
     _, H, r = q_lat.shape
     bs = rows.shape[1]
@@ -217,10 +220,11 @@ def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n:
     for t0 in range(0, n, GEMM_Q_BLOCK):
         t1 = min(n, t0 + GEMM_Q_BLOCK)
         Lb = min(nb * bs, (L - n + t1 + 7) // 8 * 8)                 # keys the block's last token sees (rows past L: weight 0)
+        k0 = max(0, L - n + t0 - window + 1) // 8 * 8 if window > 0 else 0      # the first key its first token sees
         q2 = torch.cat([q_lat[t0:t1], q_rot[t0:t1]], -1).reshape((t1 - t0) * H, -1)
-        sc = _mm_f32(q2, kv[:Lb].t()).contiguous()
-        hi, lo = _ops().sm_causal_softmax(sc, pos[t0:t1].contiguous(), H, scale, f32)
-        c = kv[:Lb, :r]
+        sc = _mm_f32(q2, kv[k0:Lb].t()).contiguous()
+        hi, lo = _ops().sm_causal_softmax(sc, pos[t0:t1].contiguous(), H, scale, f32, k0, window)
+        c = kv[k0:Lb, :r]
         o = _mm_f32(hi, c)
         if not f32:
             o += _mm_f32(lo, c)
@@ -228,7 +232,8 @@ def _latent_attention_gemm(q_lat, q_rot, rows, table_row, pos, scale, L: int, n:
     return out
 
 
-def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, gate, q_lens, ctx_lens, out_dtype):
+def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, gate, q_lens, ctx_lens, out_dtype,
+                          window: int = 0):
     T, H, r = q_lat.shape
     f32 = out_dtype == torch.float32
     # sizes the flash kernel cannot hold in LDS / registers: every portion takes the library-product path
@@ -236,13 +241,13 @@ def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, 
     big = [b for b, n in enumerate(q_lens) if n >= min_q]
     if not big:
         return _ops().sm_latent_attention(q_lat.contiguous(), q_rot, rows, block_tables, seq_of, pos, scale, gate,
-                                          max(ctx_lens), f32)
+                                          max(ctx_lens), f32, window)
     out = torch.empty(T, H, r, dtype=out_dtype, device=q_lat.device)
     small, small_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
         if n >= min_q:
             o = _latent_attention_gemm(q_lat[t0:t0 + n], q_rot[t0:t0 + n], rows, block_tables[b], pos[t0:t0 + n], scale,
-                                       L, n)
+                                       L, n, window)
             if gate is not None:
                 o = o * torch.sigmoid(gate[t0:t0 + n].float())[..., None]
             out[t0:t0 + n] = o.to(out_dtype)
@@ -254,7 +259,7 @@ def _latent_attention_gpu(q_lat, q_rot, rows, block_tables, seq_of, pos, scale, 
         idx = torch.cat(small)
         o = _ops().sm_latent_attention(q_lat[idx].contiguous(), q_rot[idx], rows, block_tables,
                                        seq_of[idx].contiguous(), pos[idx].contiguous(), scale,
-                                       gate[idx] if gate is not None else None, small_ctx, f32)
+                                       gate[idx] if gate is not None else None, small_ctx, f32, window)
         out[idx] = o
     return out
 
@@ -426,6 +431,24 @@ def head_rms_gate(h: torch.Tensor, norm_w: torch.Tensor, gate_pre: torch.Tensor,
 
 
 # ------------------------------------------------------------------ feed-forward
+GLU_ACTS = {"gelu_tanh": 0, "relu": 1, "silu": 2}
+
+
+def glu_act(gu: torch.Tensor, act: str) -> torch.Tensor:
+    """[T, 2 I] = [gate | up] -> act(gate) * up  [T, I] (f32 math), ``act`` a key of ``GLU_ACTS``."""
+    I = gu.shape[-1] // 2
+    if native(gu):
+        return _ops().sm_glu_act(gu.contiguous(), GLU_ACTS[act])
+    g, u = gu[..., :I].float(), gu[..., I:].float()
+    if act == "relu":
+        a = torch.relu(g)
+    elif act == "silu":
+        a = F.silu(g)
+    else:
+        a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+    return (a * u).to(gu.dtype)
+
+
 def glu_gelu(gu: torch.Tensor) -> torch.Tensor:
     """[T, 2 I] = [gate | up] -> gelu_tanh(gate) * up  [T, I] (f32 math)."""
     I = gu.shape[-1] // 2
