@@ -171,7 +171,18 @@ def main():
     ap.add_argument("--blockmix-sizes", default="small,base")
     ap.add_argument("--blockmix-prompts", default="1024,4096")
     ap.add_argument("--no-blockmix-ref", action="store_true", help="--blockmix: skip the comparison model")
+    ap.add_argument("--prenorm", action="store_true",
+                    help="side benchmark (not the headline metric): prefill / decode throughput of the pre-norm hybrid "
+                         "decoder (chunked attention with a sink, state-space mixer, windowed latent attention) beside "
+                         "the latent-attention + mLSTM hybrid at equal sizes, one GPU")
+    ap.add_argument("--prenorm-sizes", default="small,base")
+    ap.add_argument("--prenorm-prompts", default="1024,4096")
+    ap.add_argument("--no-prenorm-ref", action="store_true", help="--prenorm: skip the comparison model")
     args = ap.parse_args()
+    if args.prenorm:
+        from ipex_llm_amd.utils.bench_prenorm import main as prenorm_main
+        prenorm_main(args)
+        return
     if args.blockmix:
         from ipex_llm_amd.utils.bench_blockmix import main as blockmix_main
         blockmix_main(args)

@@ -33,10 +33,10 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
                       void* out, float* part, int nsplit, int T, int H, int G, int d, int dv, hipStream_t st);
 
 // rows [R, L] of raw scores of whole chunks (row i: head (i / (rep L)) % G * rep + i % rep, token (i / rep) % L of
-// its chunk, which sees keys 0 .. token): scaled, softmax with the head's sink; bf16: weights leave as hi + lo bf16
-// pairs, f32 (hi == null): in place
-void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hi,
-                   void* lo, hipStream_t st);
+// its chunk, which sees keys 0 .. token): scaled, softmax with the head's sink; bf16: the f32 weights leave as bf16
+// pairs hi + lo in hl [R, 2 L] (a row's hi halves, then its lo halves); f32 (hl == null): in place
+void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hl,
+                   hipStream_t st);
 
 // o[t, c] *= sigmoid(g[t, c]); g rows of g_ld elements
 void sigmoid_gate(bool bf16, void* o, const void* g, int64_t g_ld, int64_t T, int C, hipStream_t st);

@@ -75,7 +75,7 @@ __device__ __forceinline__ float normed(const E* x, int i, int head, int d, cons
 }
 
 template <typename E>
-__global__ void __launch_bounds__(256) qkv_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
+__global__ void __launch_bounds__(1024) qkv_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
                                                   int64_t k_ld, const E* __restrict__ v, int64_t v_ld,
                                                   const E* __restrict__ qn, const E* __restrict__ kn, bool whole,
                                                   float eps, const float* __restrict__ table, int dims, int layout,
@@ -307,34 +307,37 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
   }
 }
 
-// merge of the key splits: part [T, H, nsplit, dv + 2] -> out [T, H, dv]
+// merge of the key splits: part [T, H, nsplit, dv + 2] -> out [T, H, dv].  One wave per (token, head): lane z
+// holds split z's (max, sum) (nsplit <= 64), the wave reduces them, then every lane sums its value columns
 template <typename E>
-__global__ void __launch_bounds__(128) masked_attn_combine_k(const float* __restrict__ part, const float* __restrict__ sink,
-                                                            E* __restrict__ out, int H, int dv, int nsplit) {
+__global__ void __launch_bounds__(64) masked_attn_combine_k(const float* __restrict__ part, const float* __restrict__ sink,
+                                                           E* __restrict__ out, int H, int dv, int nsplit) {
+  __shared__ float wz[64];
   const int64_t th = (int64_t)blockIdx.x * H + blockIdx.y;
   const float* pp = part + th * nsplit * (dv + 2);
-  float M = sink ? sink[blockIdx.y] : -INFINITY;
-  for (int z = 0; z < nsplit; z++) M = fmaxf(M, pp[(size_t)z * (dv + 2) + dv]);
-  float L = sink ? expf(sink[blockIdx.y] - M) : 0.f;
-  for (int z = 0; z < nsplit; z++) {
-    const float mz = pp[(size_t)z * (dv + 2) + dv];
-    if (mz != -INFINITY) L += pp[(size_t)z * (dv + 2) + dv + 1] * expf(mz - M);
-  }
-  for (int c = threadIdx.x; c < dv; c += blockDim.x) {
+  const int lane = threadIdx.x;
+  const float mz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv] : -INFINITY;
+  const float lz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
+  const float sk = sink ? sink[blockIdx.y] : -INFINITY;
+  const float M = fmaxf(wave_max(mz), sk);
+  const float f = mz == -INFINITY ? 0.f : expf(mz - M);
+  wz[lane] = f;
+  // the splits' sums in index order (a fixed order, whatever the lanes do)
+  __syncthreads();
+  float L = sink ? expf(sk - M) : 0.f;
+  for (int z = 0; z < nsplit; z++) L += __shfl(lz, z, 64) * wz[z];
+  const float inv = 1.0f / L;
+  for (int c = lane; c < dv; c += 64) {
     float O = 0.f;
-    for (int z = 0; z < nsplit; z++) {
-      const float mz = pp[(size_t)z * (dv + 2) + dv];
-      if (mz != -INFINITY) O += pp[(size_t)z * (dv + 2) + c] * expf(mz - M);
-    }
-    stf(out + th * dv + c, O / L);
+    for (int z = 0; z < nsplit; z++) O = fmaf(pp[(size_t)z * (dv + 2) + c], wz[z], O);
+    stf(out + th * dv + c, O * inv);
   }
 }
 
 // ------------------------------------------------------------------ softmax between the chunk products
 template <typename E>
 __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, int L, int G, int rep, float scale,
-                                                      const float* __restrict__ sink, E* __restrict__ hi,
-                                                      E* __restrict__ lo) {
+                                                      const float* __restrict__ sink, E* __restrict__ hi) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
   const int tok = (int)((row / rep) % L);
@@ -358,10 +361,10 @@ __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, i
   const float inv = 1.0f / (block_sum(sum, red) + (sink ? expf(sk - mx) : 0.f));
   for (int j = threadIdx.x; j < L; j += blockDim.x) {
     const float w = j < nk ? s[j] * inv : 0.f;
-    if (hi) {
+    if (hi) {                                                      // [R, 2 L]: hi halves, then lo halves
       const E hv = (E)w;
-      hi[row * L + j] = hv;
-      lo[row * L + j] = (E)(w - (float)hv);
+      hi[row * 2 * L + j] = hv;
+      hi[row * 2 * L + L + j] = (E)(w - (float)hv);
     } else {
       s[j] = w;
     }
@@ -395,12 +398,15 @@ void qkv_norm_rope_store(bool bf16, const void* q, int64_t q_ld, const void* k, 
   (void)num_rows;
   if (T <= 0) return;
   const size_t lds = (size_t)(H + G + 2) * sizeof(float);
+  // few tokens (decode): a thread per value or two, so that no thread walks a chain of dependent loads
+  const int64_t vals = (int64_t)(H + G) * d;
+  const int nt = T > 64 ? 256 : (vals >= 1024 ? 1024 : (int)((vals + 63) / 64 * 64));
   if (bf16)
-    qkv_store_k<__bf16><<<T, 256, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)v, v_ld,
+    qkv_store_k<__bf16><<<T, nt, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)v, v_ld,
                                              (const __bf16*)qn, (const __bf16*)kn, whole, eps, table, dims, layout, pos,
                                              slots, (__bf16*)rows, qo, H, G, d, dv);
   else
-    qkv_store_k<float><<<T, 256, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
+    qkv_store_k<float><<<T, nt, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
                                             (const float*)qn, (const float*)kn, whole, eps, table, dims, layout, pos,
                                             slots, (float*)rows, qo, H, G, d, dv);
 }
@@ -463,16 +469,16 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
 #undef MA_RC
 #undef MA_LAUNCH
   if (nsplit > 1) {
-    if (bf16) masked_attn_combine_k<__bf16><<<dim3(T, H), 128, 0, st>>>(part, sink, (__bf16*)out, H, dv, nsplit);
-    else masked_attn_combine_k<float><<<dim3(T, H), 128, 0, st>>>(part, sink, (float*)out, H, dv, nsplit);
+    if (bf16) masked_attn_combine_k<__bf16><<<dim3(T, H), 64, 0, st>>>(part, sink, (__bf16*)out, H, dv, nsplit);
+    else masked_attn_combine_k<float><<<dim3(T, H), 64, 0, st>>>(part, sink, (float*)out, H, dv, nsplit);
   }
 }
 
-void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hi,
-                   void* lo, hipStream_t st) {
+void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hl,
+                   hipStream_t st) {
   if (R <= 0 || L <= 0) return;
-  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (__bf16*)hi, (__bf16*)lo);
-  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (float*)nullptr, (float*)nullptr);
+  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (__bf16*)hl);
+  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (float*)nullptr);
 }
 
 void sigmoid_gate(bool bf16, void* o, const void* g, int64_t g_ld, int64_t T, int C, hipStream_t st) {

@@ -12,7 +12,9 @@
 //                      their softplus and the decays computed once per chunk);
 //                      every wave leaves a partial y per token and the partials
 //                      are summed in a fixed order, so a result never depends
-//                      on how the tokens were cut into steps
+//                      on how the tokens were cut into steps.  The rows per
+//                      wave (8 .. 64) are chosen so that the launch fills the
+//                      chip: few sequences and heads -> more, thinner waves
 //   gated group norm   y silu(z), every group divided by its root mean square
 //
 // Activations are bf16 or f32 (template E); accumulation is always f32.
@@ -106,7 +108,7 @@ __global__ void __launch_bounds__(256) conv_state_k(const E* __restrict__ u, int
 
 // ------------------------------------------------------------------ scan
 template <typename E, int NS>
-__global__ void __launch_bounds__(NS == 64 ? 1024 : 256) scan_k(
+__global__ void __launch_bounds__(1024) scan_k(
     const float* __restrict__ x, int64_t x_ld, const float* __restrict__ Bm, int64_t b_ld, const float* __restrict__ Cm,
     int64_t c_ld, const E* __restrict__ dtp, int64_t dt_ld, const float* __restrict__ dt_bias,
     const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ S,
@@ -159,28 +161,43 @@ __global__ void __launch_bounds__(NS == 64 ? 1024 : 256) scan_k(
       const float dx = ds[tk] * xs[tk * 64 + lane];
       const float4* b4 = (const float4*)(Bs + (size_t)tk * NP + wv * NS);
       const float4* c4 = (const float4*)(Cs + (size_t)tk * NP + wv * NS);
-      float acc = 0.f;
+      // y's sum over the state rows has one fixed shape, whatever NS is: units of 8 rows (four chains of two),
+      // then a balanced pairwise tree over the units -- here over the wave's units, below over the waves
+      float un[NS / 8];
 #pragma unroll
-      for (int i = 0; i < NS / 4; i++) {
-        const float4 bv = b4[i], cv = c4[i];
-        st[4 * i + 0] = fmaf(da, st[4 * i + 0], dx * bv.x);
-        st[4 * i + 1] = fmaf(da, st[4 * i + 1], dx * bv.y);
-        st[4 * i + 2] = fmaf(da, st[4 * i + 2], dx * bv.z);
-        st[4 * i + 3] = fmaf(da, st[4 * i + 3], dx * bv.w);
-        acc = fmaf(st[4 * i + 0], cv.x, acc);
-        acc = fmaf(st[4 * i + 1], cv.y, acc);
-        acc = fmaf(st[4 * i + 2], cv.z, acc);
-        acc = fmaf(st[4 * i + 3], cv.w, acc);
+      for (int u = 0; u < NS / 8; u++) {
+        const float4 b0 = b4[2 * u], b1 = b4[2 * u + 1], c0v = c4[2 * u], c1v = c4[2 * u + 1];
+        float* r = st + 8 * u;
+        r[0] = fmaf(da, r[0], dx * b0.x);
+        r[1] = fmaf(da, r[1], dx * b0.y);
+        r[2] = fmaf(da, r[2], dx * b0.z);
+        r[3] = fmaf(da, r[3], dx * b0.w);
+        r[4] = fmaf(da, r[4], dx * b1.x);
+        r[5] = fmaf(da, r[5], dx * b1.y);
+        r[6] = fmaf(da, r[6], dx * b1.z);
+        r[7] = fmaf(da, r[7], dx * b1.w);
+        const float a0 = fmaf(r[4], c1v.x, r[0] * c0v.x), a1 = fmaf(r[5], c1v.y, r[1] * c0v.y);
+        const float a2 = fmaf(r[6], c1v.z, r[2] * c0v.z), a3 = fmaf(r[7], c1v.w, r[3] * c0v.w);
+        un[u] = (a0 + a1) + (a2 + a3);
       }
-      pt[((size_t)wv * TC + tk) * 64 + lane] = acc;
+#pragma unroll
+      for (int sft = 1; sft < NS / 8; sft *= 2)
+#pragma unroll
+        for (int u = 0; u + sft < NS / 8; u += 2 * sft) un[u] += un[u + sft];
+      pt[((size_t)wv * TC + tk) * 64 + lane] = un[0];
     }
     __syncthreads();
     for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
       const int tk = i >> 6, l = i & 63;
       if (p0 + l >= P) continue;
-      float y = 0.f;
-      for (int w = 0; w < NW; w++) y += pt[((size_t)w * TC + tk) * 64 + l];
-      out[((int64_t)(t0 + c0 + tk) * H + h) * P + p0 + l] = fmaf(dsk, xs[i], y);
+      float v[16];                                                  // the waves' partials, zeros past NW
+#pragma unroll
+      for (int w = 0; w < 16; w++) v[w] = w < NW ? pt[((size_t)w * TC + tk) * 64 + l] : 0.f;
+#pragma unroll
+      for (int sft = 1; sft < 16; sft *= 2)
+#pragma unroll
+        for (int w = 0; w + sft < 16; w += 2 * sft) v[w] += v[w + sft];
+      out[((int64_t)(t0 + c0 + tk) * H + h) * P + p0 + l] = fmaf(dsk, xs[i], v[0]);
     }
   }
 #pragma unroll
@@ -233,7 +250,17 @@ void selective_scan(bool bf16, const float* x, int64_t x_ld, const float* Bm, in
                     const float* d_skip, float* S, const int32_t* cu, const int32_t* slots, const int64_t* pos,
                     float* out, int B, int H, int P, int G, int N, hipStream_t st) {
   if (B <= 0 || N > kScanMaxState) return;                          // (sizes are refused by the caller beforehand)
-  const int NS = N <= 64 ? 16 : (N <= 128 ? 32 : 64);
+  // state rows per wave: as few as fill the chip -- the scan is sequential in time, so its only parallelism is
+  // (sequence, head, 64 columns, wave); at most 16 waves a workgroup
+  const int64_t cols = (int64_t)B * H * ((P + 63) / 64);
+  int NS = 64;
+  for (int ns = 8; ns <= 64; ns *= 2) {
+    const int nw = (N + ns - 1) / ns;
+    if (nw <= 16 && (ns == 64 || cols * ((N + 2 * ns - 1) / (2 * ns)) < 2048)) {
+      NS = ns;
+      break;
+    }
+  }
   const int NW = (N + NS - 1) / NS;
   const int NP = NW * NS;
   // tokens per chunk: B and C rows, x, the waves' partials and the step sizes within 48 KB
@@ -245,11 +272,13 @@ void selective_scan(bool bf16, const float* x, int64_t x_ld, const float* Bm, in
   scan_k<E, NSV><<<grid, block, lds, st>>>(x, x_ld, Bm, b_ld, Cm, c_ld, (const E*)dt, dt_ld, dt_bias, a_log, d_skip, S, \
                                            cu, slots, pos, out, H, P, G, N, TC)
   if (bf16) {
-    if (NS == 16) SSM_SCAN(__bf16, 16);
+    if (NS == 8) SSM_SCAN(__bf16, 8);
+    else if (NS == 16) SSM_SCAN(__bf16, 16);
     else if (NS == 32) SSM_SCAN(__bf16, 32);
     else SSM_SCAN(__bf16, 64);
   } else {
-    if (NS == 16) SSM_SCAN(float, 16);
+    if (NS == 8) SSM_SCAN(float, 8);
+    else if (NS == 16) SSM_SCAN(float, 16);
     else if (NS == 32) SSM_SCAN(float, 32);
     else SSM_SCAN(float, 64);
   }

@@ -128,8 +128,9 @@ int64_t ma_masked_attention_fits(bool bf16, int64_t rep, int64_t d, int64_t dv) 
   return illm::ma::masked_attention_plan(bf16, (int)rep, (int)d, (int)dv, &nw, &hb);
 }
 
-// scores f32 [R, L] of whole chunks -> softmax weights with the sink; bf16 pair (hi, lo) or in place (f32)
-std::tuple<Tensor, Tensor> ma_chunk_softmax(Tensor& scores, int64_t G, int64_t rep, double scale,
+// scores f32 [R, L] of whole chunks -> softmax weights with the sink: bf16 [R, 2 L] (hi halves | lo halves), or in
+// place (f32)
+Tensor ma_chunk_softmax(Tensor& scores, int64_t G, int64_t rep, double scale,
                                             const c10::optional<Tensor>& sink, bool act_f32) {
   c10::DeviceGuard g(scores.device());
   TORCH_CHECK(scores.is_cuda() && scores.dim() == 2 && scores.scalar_type() == at::kFloat && scores.is_contiguous(),
@@ -142,15 +143,11 @@ std::tuple<Tensor, Tensor> ma_chunk_softmax(Tensor& scores, int64_t G, int64_t r
                 "ma_chunk_softmax: sink f32 [H]");
     sk = sink->data_ptr<float>();
   }
-  Tensor hi, lo;
-  if (!act_f32) {
-    hi = at::empty({R, L}, scores.options().dtype(at::kBFloat16));
-    lo = at::empty({R, L}, scores.options().dtype(at::kBFloat16));
-  }
+  Tensor hl;
+  if (!act_f32) hl = at::empty({R, 2 * L}, scores.options().dtype(at::kBFloat16));
   illm::ma::chunk_softmax(!act_f32, scores.data_ptr<float>(), R, (int)L, (int)G, (int)rep, (float)scale, sk,
-                          act_f32 ? nullptr : hi.data_ptr(), act_f32 ? nullptr : lo.data_ptr(), stream());
-  if (act_f32) return {scores, scores};
-  return {hi, lo};
+                          act_f32 ? nullptr : hl.data_ptr(), stream());
+  return act_f32 ? scores : hl;
 }
 
 Tensor ma_sigmoid_gate(Tensor& o, const Tensor& gate) {
@@ -172,7 +169,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("ma_masked_attention(Tensor q, Tensor rows, int G, int dv, Tensor block_tables, Tensor seq_of, Tensor pos, "
         "float scale, int mask, int size, Tensor? sink, int max_ctx, bool act_f32) -> Tensor");
   m.def("ma_masked_attention_fits(bool bf16, int rep, int d, int dv) -> int");
-  m.def("ma_chunk_softmax(Tensor(a!) scores, int G, int rep, float scale, Tensor? sink, bool act_f32) -> (Tensor, Tensor)");
+  m.def("ma_chunk_softmax(Tensor(a!) scores, int G, int rep, float scale, Tensor? sink, bool act_f32) -> Tensor");
   m.def("ma_sigmoid_gate(Tensor(a!) o, Tensor gate) -> Tensor(a!)");
 }
 

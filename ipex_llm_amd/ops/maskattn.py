@@ -20,7 +20,7 @@ from typing import List, Optional
 
 import torch
 
-from .seqmix import native, _mm_f32
+from .seqmix import native
 
 __all__ = ["MASKS", "LAYOUTS", "first_visible", "qkv_norm_rope_store", "masked_attention", "sigmoid_gate"]
 
@@ -174,16 +174,16 @@ def _chunk_blocks_gemm(q, rows, table_row, G, dv, scale, size, sink, t0, c0, nc,
     qq = q[t0:t0 + n].view(nc, size, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, size * rep, d)
     if f32:
         sc = torch.bmm(qq, kk)
-    else:                                       # f32 queries against 16-bit keys: hi + lo halves of q
-        qh = qq.to(rows.dtype)
-        ql = (qq - qh.float()).to(rows.dtype)
-        sc = torch.bmm(qh, kk, out_dtype=torch.float32) + torch.bmm(ql, kk, out_dtype=torch.float32)
-    hi, lo_w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, f32)
-    hi = hi.view(nc * G, size * rep, size)
-    if f32:
-        o = torch.bmm(hi, vv)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, True)
+        o = torch.bmm(w.view(nc * G, size * rep, size), vv)
     else:
-        o = torch.bmm(hi, vv, out_dtype=torch.float32) + torch.bmm(lo_w.view_as(hi), vv, out_dtype=torch.float32)
+        # f32 queries against 16-bit keys, f32 weights against 16-bit values: hi + lo halves side by side along the
+        # summed axis, the keys / values twice, so each product is one launch with f32 accumulation
+        qh = qq.to(rows.dtype)
+        q2 = torch.cat([qh, (qq - qh.float()).to(rows.dtype)], -1)
+        sc = torch.bmm(q2, torch.cat([kk, kk], 1), out_dtype=torch.float32)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, False)
+        o = torch.bmm(w.view(nc * G, size * rep, 2 * size), torch.cat([vv, vv], 1), out_dtype=torch.float32)
     o = o.view(nc, G, size, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
     out[t0:t0 + n] = o.to(out.dtype)
 
