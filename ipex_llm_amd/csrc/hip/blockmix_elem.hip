@@ -74,7 +74,31 @@ __global__ void __launch_bounds__(1024) add_rms_norm_k(float* __restrict__ x, co
   }
 }
 
-// x += y (y may be null), then out = x / sqrt(mean(x^2) + eps) * w: one sublayer's residual sum and the next norm
+// four consecutive values as one access
+template <typename E> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void ld(const float* p, float* v) {
+    const float4 a = *(const float4*)p;
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+  }
+  static __device__ __forceinline__ void st(float* p, const float* v) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4<__bf16> {
+  typedef __bf16 B4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ void ld(const __bf16* p, float* v) {
+    const B4 a = *(const B4*)p;
+    v[0] = (float)a[0], v[1] = (float)a[1], v[2] = (float)a[2], v[3] = (float)a[3];
+  }
+  static __device__ __forceinline__ void st(__bf16* p, const float* v) {
+    B4 a;
+    a[0] = (__bf16)v[0], a[1] = (__bf16)v[1], a[2] = (__bf16)v[2], a[3] = (__bf16)v[3];
+    *(B4*)p = a;
+  }
+};
+
+// x += y (y may be null), then out = x / sqrt(mean(x^2) + eps) * w: one sublayer's residual sum and the next norm.
+// Rows whose length is a multiple of 4 move as 4-value accesses and stay in registers between the two passes
+// (up to 16 values a thread; longer rows read the rest back).
 template <typename E>
 __global__ void __launch_bounds__(1024) add_rms_norm_rows_k(float* __restrict__ x, const E* __restrict__ y,
                                                           const E* __restrict__ w, E* __restrict__ out, int W, float eps) {
@@ -82,6 +106,62 @@ __global__ void __launch_bounds__(1024) add_rms_norm_rows_k(float* __restrict__ 
   const int64_t t = blockIdx.x;
   float* xr = x + t * W;
   float q = 0.f;
+  if ((W & 3) == 0) {
+    const int W4 = W >> 2, bd = blockDim.x;
+    float keep[4][4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const int c = 4 * (threadIdx.x + k * bd);
+      if (c < W) {
+        float v[4], a[4];
+        Vec4<float>::ld(xr + c, v);
+        if (y) {
+          Vec4<E>::ld(y + t * W + c, a);
+#pragma unroll
+          for (int i = 0; i < 4; i++) v[i] += a[i];
+          Vec4<float>::st(xr + c, v);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          keep[k][i] = v[i];
+          q += v[i] * v[i];
+        }
+      }
+    }
+    for (int c4 = threadIdx.x + 4 * bd; c4 < W4; c4 += bd) {
+      float v[4], a[4];
+      Vec4<float>::ld(xr + 4 * c4, v);
+      if (y) {
+        Vec4<E>::ld(y + t * W + 4 * c4, a);
+#pragma unroll
+        for (int i = 0; i < 4; i++) v[i] += a[i];
+        Vec4<float>::st(xr + 4 * c4, v);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++) q += v[i] * v[i];
+    }
+    const float rs = 1.0f / sqrtf(block_sum(q, red) / (float)W + eps);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const int c = 4 * (threadIdx.x + k * bd);
+      if (c < W) {
+        float g[4], o[4];
+        Vec4<E>::ld(w + c, g);
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = keep[k][i] * rs * g[i];
+        Vec4<E>::st(out + t * W + c, o);
+      }
+    }
+    for (int c4 = threadIdx.x + 4 * bd; c4 < W4; c4 += bd) {
+      float v[4], g[4], o[4];
+      Vec4<float>::ld(xr + 4 * c4, v);                              // own writes
+      Vec4<E>::ld(w + 4 * c4, g);
+#pragma unroll
+      for (int i = 0; i < 4; i++) o[i] = v[i] * rs * g[i];
+      Vec4<E>::st(out + t * W + 4 * c4, o);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float v = xr[c];
     if (y) {

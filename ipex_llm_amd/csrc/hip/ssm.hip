@@ -136,26 +136,58 @@ __global__ void __launch_bounds__(1024) scan_k(
     st[i] = (!fresh && nn < N && pc < P) ? Sg[(int64_t)nn * P + pc] : 0.f;
   }
   const float rate = expf(a_log[h]), bias = dt_bias[h], dsk = d_skip[h];
+  // a chunk's B / C / x / dt elements travel global -> registers -> LDS; the registers of the NEXT chunk are
+  // requested before the current chunk's arithmetic, so their latency hides behind it (the host sizes TC so that
+  // PE elements per thread and array cover a chunk)
+  constexpr int PE = 4;
+  float rb[PE], rc[PE], rx[PE], rdt = 0.f;
+  auto fetch = [&](int c0) {
+    const int nt = min(TC, n - c0);
+#pragma unroll
+    for (int k = 0; k < PE; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      rb[k] = rc[k] = 0.f;
+      if (i < nt * NP) {
+        const int tk = i / NP, nn = i - tk * NP;
+        const int64_t t = t0 + c0 + tk;
+        if (nn < N) {
+          rb[k] = Bm[t * b_ld + (int64_t)g * N + nn];
+          rc[k] = Cm[t * c_ld + (int64_t)g * N + nn];
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < PE; k++) {
+      const int i = threadIdx.x + k * blockDim.x;                   // (token i / 64, this lane's column)
+      rx[k] = (i < nt * 64 && pc < P) ? x[(int64_t)(t0 + c0 + (i >> 6)) * x_ld + (int64_t)h * P + pc] : 0.f;
+    }
+    if (threadIdx.x < nt) rdt = ldf(dtp + (int64_t)(t0 + c0 + threadIdx.x) * dt_ld + h);
+  };
+  fetch(0);
   for (int c0 = 0; c0 < n; c0 += TC) {
     const int nt = min(TC, n - c0);
     __syncthreads();                                                // the last chunk's reads are done
-    for (int i = threadIdx.x; i < nt * NP; i += blockDim.x) {
-      const int tk = i / NP, nn = i - tk * NP;
-      const int64_t t = t0 + c0 + tk;
-      Bs[i] = nn < N ? Bm[t * b_ld + (int64_t)g * N + nn] : 0.f;
-      Cs[i] = nn < N ? Cm[t * c_ld + (int64_t)g * N + nn] : 0.f;
+#pragma unroll
+    for (int k = 0; k < PE; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      if (i < nt * NP) {
+        Bs[i] = rb[k];
+        Cs[i] = rc[k];
+      }
     }
-    for (int i = threadIdx.x; i < nt * 64; i += blockDim.x) {
-      const int tk = i >> 6, l = i & 63;
-      xs[i] = p0 + l < P ? x[(int64_t)(t0 + c0 + tk) * x_ld + (int64_t)h * P + p0 + l] : 0.f;
+#pragma unroll
+    for (int k = 0; k < PE; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      if (i < nt * 64) xs[i] = rx[k];
     }
     if (threadIdx.x < nt) {
-      const float z = ldf(dtp + (int64_t)(t0 + c0 + threadIdx.x) * dt_ld + h) + bias;
+      const float z = rdt + bias;
       const float dt = z > 20.f ? z : log1pf(expf(z));              // softplus
       ds[threadIdx.x] = dt;
       ds[TC + threadIdx.x] = expf(-rate * dt);
     }
     __syncthreads();
+    if (c0 + TC < n) fetch(c0 + TC);
     for (int tk = 0; tk < nt; tk++) {
       const float da = ds[TC + tk];
       const float dx = ds[tk] * xs[tk * 64 + lane];
@@ -263,9 +295,13 @@ void selective_scan(bool bf16, const float* x, int64_t x_ld, const float* Bm, in
   }
   const int NW = (N + NS - 1) / NS;
   const int NP = NW * NS;
-  // tokens per chunk: B and C rows, x, the waves' partials and the step sizes within 48 KB
+  // tokens per chunk: B and C rows, x, the waves' partials and the step sizes within 48 KB; a thread stages at most
+  // four elements of B, of C and of x per chunk (4 * 64 NW >= TC * NP and >= 64 TC)
   int TC = (48 * 1024 / 4) / (2 * NP + 64 + NW * 64 + 2);
-  TC = TC > 16 ? 16 : (TC < 1 ? 1 : TC);
+  TC = TC > 16 ? 16 : TC;
+  TC = TC > 256 / NS ? 256 / NS : TC;
+  TC = TC > 4 * NW ? 4 * NW : TC;
+  TC = TC < 1 ? 1 : TC;
   const size_t lds = ((size_t)TC * (2 * NP + 64 + NW * 64) + 2 * TC) * sizeof(float);
   dim3 grid(B, H, (P + 63) / 64), block(64 * NW);
 #define SSM_SCAN(E, NSV)                                                                                              \

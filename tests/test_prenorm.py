@@ -102,17 +102,18 @@ def test_add_norm_and_gates(dev):
     from ipex_llm_amd.ops import blockmix as BM, maskattn as MA, seqmix as SM, ssm as SSM
     g = torch.Generator().manual_seed(0)
     for act in (torch.float32, torch.bfloat16):
-        x = torch.randn(7, 50, generator=g)
-        y = torch.randn(7, 50, generator=g).to(act)
-        w = (1 + 0.3 * torch.randn(50, generator=g)).to(act)
-        xs = x.clone().to(dev)
-        h = BM.add_rms_norm_rows_(xs, y.to(dev), w.to(dev), 1e-5, act)
-        s = x.double() + y.double()
-        assert torch.equal(xs.cpu(), (x + y.float()))
-        want = O.unit_rms(s, 1e-5) * w.double()
-        assert h.dtype == act and (h.double().cpu() - want).abs().max() < (1e-5 if act == torch.float32 else 3e-2)
-        h0 = BM.add_rms_norm_rows_(xs, None, w.to(dev), 1e-5, act)          # nothing to add: a plain norm
-        assert (h0.double().cpu() - want).abs().max() < (1e-5 if act == torch.float32 else 3e-2)
+        for T, Wd in ((7, 50), (7, 52), (70, 4160)):                        # odd rows, 4-value rows, rows past the registers
+            x = torch.randn(T, Wd, generator=g)
+            y = torch.randn(T, Wd, generator=g).to(act)
+            w = (1 + 0.3 * torch.randn(Wd, generator=g)).to(act)
+            xs = x.clone().to(dev)
+            h = BM.add_rms_norm_rows_(xs, y.to(dev), w.to(dev), 1e-5, act)
+            s = x.double() + y.double()
+            assert torch.equal(xs.cpu(), (x + y.float()))
+            want = O.unit_rms(s, 1e-5) * w.double()
+            assert h.dtype == act and (h.double().cpu() - want).abs().max() < (2e-5 if act == torch.float32 else 5e-2)
+            h0 = BM.add_rms_norm_rows_(xs, None, w.to(dev), 1e-5, act)      # nothing to add: a plain norm
+            assert (h0.double().cpu() - want).abs().max() < (2e-5 if act == torch.float32 else 5e-2)
         gu = torch.randn(5, 2 * 33, generator=g).to(act)
         for name, f in (("relu", torch.relu), ("silu", O.silu), ("gelu_tanh", None)):
             a = gu[:, :33].double()
