@@ -32,11 +32,12 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
                       const int32_t* seq_of, const int64_t* pos, float scale, int mask, int size, const float* sink,
                       void* out, float* part, int nsplit, int T, int H, int G, int d, int dv, hipStream_t st);
 
-// rows [R, L] of raw scores of whole chunks (row i: head (i / (rep L)) % G * rep + i % rep, token (i / rep) % L of
-// its chunk, which sees keys 0 .. token): scaled, softmax with the head's sink; bf16: the f32 weights leave as bf16
-// pairs hi + lo in hl [R, 2 L] (a row's hi halves, then its lo halves); f32 (hl == null): in place
-void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hl,
-                   hipStream_t st);
+// rows [R, L] of raw scores of pieces of chunks: a piece is L keys from a chunk's first position on, its queries are
+// its last Lq positions (Lq == L: a whole chunk).  Row i: head (i / (rep Lq)) % G * rep + i % rep, query
+// (i / rep) % Lq, which sees keys 0 .. L - Lq + query.  Scaled, softmax with the head's sink; bf16: the f32 weights
+// leave as bf16 pairs hi + lo in hl [R, 2 L] (a row's hi halves, then its lo halves); f32 (hl == null): in place
+void chunk_softmax(bool bf16, float* sc, int64_t R, int Lq, int L, int G, int rep, float scale, const float* sink,
+                   void* hl, hipStream_t st);
 
 // o[t, c] *= sigmoid(g[t, c]); g rows of g_ld elements
 void sigmoid_gate(bool bf16, void* o, const void* g, int64_t g_ld, int64_t T, int C, hipStream_t st);

@@ -336,13 +336,13 @@ __global__ void __launch_bounds__(64) masked_attn_combine_k(const float* __restr
 
 // ------------------------------------------------------------------ softmax between the chunk products
 template <typename E>
-__global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, int L, int G, int rep, float scale,
+__global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, int Lq, int L, int G, int rep, float scale,
                                                       const float* __restrict__ sink, E* __restrict__ hi) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
-  const int tok = (int)((row / rep) % L);
-  const int h = (int)((row / ((int64_t)rep * L)) % G) * rep + (int)(row % rep);
-  const int nk = tok + 1;
+  const int tok = (int)((row / rep) % Lq);                          // the piece's queries are its last Lq positions
+  const int h = (int)((row / ((int64_t)rep * Lq)) % G) * rep + (int)(row % rep);
+  const int nk = L - Lq + tok + 1;
   float* s = sc + row * L;
   const float sk = sink ? sink[h] : -INFINITY;
   float mx = sk;
@@ -474,11 +474,11 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
   }
 }
 
-void chunk_softmax(bool bf16, float* sc, int64_t R, int L, int G, int rep, float scale, const float* sink, void* hl,
-                   hipStream_t st) {
+void chunk_softmax(bool bf16, float* sc, int64_t R, int Lq, int L, int G, int rep, float scale, const float* sink,
+                   void* hl, hipStream_t st) {
   if (R <= 0 || L <= 0) return;
-  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (__bf16*)hl);
-  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, L, G, rep, scale, sink, (float*)nullptr);
+  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (__bf16*)hl);
+  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (float*)nullptr);
 }
 
 void sigmoid_gate(bool bf16, void* o, const void* g, int64_t g_ld, int64_t T, int C, hipStream_t st) {

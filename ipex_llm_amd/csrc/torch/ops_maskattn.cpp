@@ -130,13 +130,14 @@ int64_t ma_masked_attention_fits(bool bf16, int64_t rep, int64_t d, int64_t dv) 
 
 // scores f32 [R, L] of whole chunks -> softmax weights with the sink: bf16 [R, 2 L] (hi halves | lo halves), or in
 // place (f32)
-Tensor ma_chunk_softmax(Tensor& scores, int64_t G, int64_t rep, double scale,
-                                            const c10::optional<Tensor>& sink, bool act_f32) {
+Tensor ma_chunk_softmax(Tensor& scores, int64_t Lq, int64_t G, int64_t rep, double scale,
+                        const c10::optional<Tensor>& sink, bool act_f32) {
   c10::DeviceGuard g(scores.device());
   TORCH_CHECK(scores.is_cuda() && scores.dim() == 2 && scores.scalar_type() == at::kFloat && scores.is_contiguous(),
               "ma_chunk_softmax: scores f32 [R, L] contiguous");
   const int64_t R = scores.size(0), L = scores.size(1);
-  TORCH_CHECK(G >= 1 && rep >= 1 && R % (G * rep * L) == 0, "ma_chunk_softmax: rows must be chunks x key heads x L x rep");
+  TORCH_CHECK(G >= 1 && rep >= 1 && Lq >= 1 && Lq <= L && R % (G * rep * Lq) == 0,
+              "ma_chunk_softmax: rows must be pieces x key heads x Lq x rep, Lq <= L");
   const float* sk = nullptr;
   if (has(sink)) {
     TORCH_CHECK(sink->is_cuda() && sink->scalar_type() == at::kFloat && sink->is_contiguous() && sink->numel() == G * rep,
@@ -145,7 +146,7 @@ Tensor ma_chunk_softmax(Tensor& scores, int64_t G, int64_t rep, double scale,
   }
   Tensor hl;
   if (!act_f32) hl = at::empty({R, 2 * L}, scores.options().dtype(at::kBFloat16));
-  illm::ma::chunk_softmax(!act_f32, scores.data_ptr<float>(), R, (int)L, (int)G, (int)rep, (float)scale, sk,
+  illm::ma::chunk_softmax(!act_f32, scores.data_ptr<float>(), R, (int)Lq, (int)L, (int)G, (int)rep, (float)scale, sk,
                           act_f32 ? nullptr : hl.data_ptr(), stream());
   return act_f32 ? scores : hl;
 }
@@ -169,7 +170,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("ma_masked_attention(Tensor q, Tensor rows, int G, int dv, Tensor block_tables, Tensor seq_of, Tensor pos, "
         "float scale, int mask, int size, Tensor? sink, int max_ctx, bool act_f32) -> Tensor");
   m.def("ma_masked_attention_fits(bool bf16, int rep, int d, int dv) -> int");
-  m.def("ma_chunk_softmax(Tensor(a!) scores, int G, int rep, float scale, Tensor? sink, bool act_f32) -> Tensor");
+  m.def("ma_chunk_softmax(Tensor(a!) scores, int Lq, int G, int rep, float scale, Tensor? sink, bool act_f32) -> Tensor");
   m.def("ma_sigmoid_gate(Tensor(a!) o, Tensor gate) -> Tensor(a!)");
 }
 

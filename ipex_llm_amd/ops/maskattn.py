@@ -102,10 +102,10 @@ def qkv_norm_rope_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[
     return qf.contiguous()
 
 
-# GPU paths by portion: decoded tokens and short or unaligned pieces run the one-pass kernel, a workgroup per
-# (token, key head).  With chunks, a portion's whole chunks (from a chunk's first position to its last) see only
-# their own keys: at least GEMM_MIN_CHUNK tokens per chunk and they run as batched library products over the
-# chunks, with the fused softmax (sink, causal mask inside the chunk) between them.
+# GPU paths by portion: decoded tokens and short pieces run the one-pass kernel, a workgroup per (token, key head).
+# With chunks, a portion splits into pieces that each see only keys of their own chunk (the rest of the chunk the
+# portion starts in, whole chunks, the start of a last chunk): pieces of at least GEMM_MIN_CHUNK queries run as
+# batched library products, with the fused softmax (sink, causal mask inside the chunk) between them.
 GEMM_MIN_CHUNK = int(os.environ.get("ILLM_MASKATTN_GEMM_MIN", "128"))
 
 
@@ -156,35 +156,36 @@ def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block
     return out.reshape(T, H * dv).to(out_dtype)
 
 
-def _chunk_blocks_gemm(q, rows, table_row, G, dv, scale, size, sink, t0, c0, nc, out):
-    """``nc`` whole chunks of one sequence, starting at chunk index ``c0`` with the step's token ``t0``: scores and
-    weighted sums as batched products over (chunk, key head), the sink softmax fused between them"""
+def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out):
+    """``nc`` pieces of chunks of one sequence: piece i holds the ``nk`` keys from position ``lo + i nk`` (a chunk's
+    first position) on, and its queries are its last ``nq`` positions (whole chunks: nq == nk == the chunk size;
+    one piece with nq < nk: a portion that starts inside a chunk); the step's token ``t0`` is the first query.
+    Scores and weighted sums are batched products over (piece, key head), the sink softmax is fused between them."""
     _, H, d = q.shape
     rep = H // G
     bs = rows.shape[1]
     f32 = rows.dtype == torch.float32
-    n = nc * size
-    lo = c0 * size
-    # the chunks' rows in position order (gathered through the block table)
-    p = torch.arange(lo, lo + n, device=q.device)
+    # the pieces' rows in position order (gathered through the block table)
+    p = torch.arange(lo, lo + nc * nk, device=q.device)
     ridx = table_row.long()[p // bs] * bs + p % bs
     kv = rows.view(-1, rows.shape[-1]).index_select(0, ridx)
-    kk = kv[:, :G * d].reshape(nc, size, G, d).permute(0, 2, 3, 1).reshape(nc * G, d, size)
-    vv = kv[:, G * d:].reshape(nc, size, G, dv).permute(0, 2, 1, 3).reshape(nc * G, size, dv)
-    qq = q[t0:t0 + n].view(nc, size, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, size * rep, d)
+    kk = kv[:, :G * d].reshape(nc, nk, G, d).permute(0, 2, 3, 1).reshape(nc * G, d, nk)
+    vv = kv[:, G * d:].reshape(nc, nk, G, dv).permute(0, 2, 1, 3).reshape(nc * G, nk, dv)
+    n = nc * nq
+    qq = q[t0:t0 + n].view(nc, nq, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, nq * rep, d)
     if f32:
         sc = torch.bmm(qq, kk)
-        w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, True)
-        o = torch.bmm(w.view(nc * G, size * rep, size), vv)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, True)
+        o = torch.bmm(w.view(nc * G, nq * rep, nk), vv)
     else:
         # f32 queries against 16-bit keys, f32 weights against 16-bit values: hi + lo halves side by side along the
         # summed axis, the keys / values twice, so each product is one launch with f32 accumulation
         qh = qq.to(rows.dtype)
         q2 = torch.cat([qh, (qq - qh.float()).to(rows.dtype)], -1)
         sc = torch.bmm(q2, torch.cat([kk, kk], 1), out_dtype=torch.float32)
-        w = _ops().ma_chunk_softmax(sc.view(nc * G * size * rep, size), G, rep, scale, sink, False)
-        o = torch.bmm(w.view(nc * G, size * rep, 2 * size), torch.cat([vv, vv], 1), out_dtype=torch.float32)
-    o = o.view(nc, G, size, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False)
+        o = torch.bmm(w.view(nc * G, nq * rep, 2 * nk), torch.cat([vv, vv], 1), out_dtype=torch.float32)
+    o = o.view(nc, G, nq, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
     out[t0:t0 + n] = o.to(out.dtype)
 
 
@@ -194,28 +195,31 @@ def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask
     f32 = out_dtype == torch.float32
     q = q.contiguous()
     code = MASKS[mask]
-    big = mask == "chunk" and size >= GEMM_MIN_CHUNK and max(q_lens) >= size and _bmm_f32_ok(rows.dtype)
+    big = mask == "chunk" and GEMM_MIN_CHUNK > 0 and max(q_lens) >= GEMM_MIN_CHUNK and _bmm_f32_ok(rows.dtype)
     if not big:
         return _ops().ma_masked_attention(q, rows, G, dv, block_tables, seq_of, pos, scale, code, size, sink,
                                           max(ctx_lens), f32)
     out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
     rest, rest_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
-        p0 = L - n                                                   # position of the portion's first token
-        c0 = -(-p0 // size)                                          # first chunk that starts inside the portion
-        nc = (L - c0 * size) // size if L >= c0 * size else 0
-        if nc > 0:
-            a = t0 + c0 * size - p0
-            _chunk_blocks_gemm(q, rows, block_tables[b], G, dv, scale, size, sink, a, c0, nc, out)
-            if a > t0:
-                rest.append(torch.arange(t0, a, device=q.device))
-            if a + nc * size < t0 + n:
-                rest.append(torch.arange(a + nc * size, t0 + n, device=q.device))
-            if a > t0 or a + nc * size < t0 + n:
+        # the portion [p0, L) falls into: the rest of the chunk it starts in, whole chunks, the start of a last chunk;
+        # each is block-diagonal, and those of at least GEMM_MIN_CHUNK queries run as products
+        p0, t = L - n, t0
+        while p0 < L:
+            c0 = p0 - p0 % size                                      # first position of p0's chunk
+            if p0 == c0 and L - p0 >= size:
+                nc = (L - p0) // size
+                nq = nk = size
+            else:
+                nc, nq = 1, min(L, c0 + size) - p0
+                nk = p0 - c0 + nq
+            if nq >= GEMM_MIN_CHUNK:
+                _pieces_gemm(q, rows, block_tables[b], G, dv, scale, sink, t, c0, nc, nk, nq, out)
+            else:
+                rest.append(torch.arange(t, t + nc * nq, device=q.device))
                 rest_ctx = max(rest_ctx, L)
-        elif n:
-            rest.append(torch.arange(t0, t0 + n, device=q.device))
-            rest_ctx = max(rest_ctx, L)
+            p0 += nc * nq
+            t += nc * nq
         t0 += n
     if rest:
         idx = torch.cat(rest)

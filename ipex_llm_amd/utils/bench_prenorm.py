@@ -24,10 +24,11 @@ import torch
 SIZES = {
     # width, vocab, ff; attention (heads, kv heads, dim, vdim, rotated dims, chunk); state-space (heads, vdim, state,
     # groups, taps, norm groups); latent attention (heads, dim, rot, vdim, rank, window); mLSTM of the comparison
-    # model (heads, dim, vdim); blocks of four layers
-    "small": dict(width=1024, vocab=32000, ff=2816, attn=(8, 2, 128, 128, 64, 1024), ssm=(32, 64, 128, 1, 4, 1),
+    # model (heads, dim, vdim); blocks of four layers.  The chunks do not divide the prompt lengths, so prompts end
+    # and decoding runs inside a chunk (256 and 1024 keys in view)
+    "small": dict(width=1024, vocab=32000, ff=2816, attn=(8, 2, 128, 128, 64, 768), ssm=(32, 64, 128, 1, 4, 1),
                   latent=(8, 64, 32, 64, 256, 1024), mlstm=(4, 64, 256), blocks=1),
-    "base": dict(width=2048, vocab=32000, ff=5632, attn=(16, 4, 128, 128, 64, 2048), ssm=(64, 64, 128, 8, 4, 8),
+    "base": dict(width=2048, vocab=32000, ff=5632, attn=(16, 4, 128, 128, 64, 1536), ssm=(64, 64, 128, 8, 4, 8),
                  latent=(16, 128, 64, 128, 512, 2048), mlstm=(4, 256, 512), blocks=1),
 }
 

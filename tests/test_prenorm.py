@@ -491,15 +491,17 @@ def test_bfloat16_serving_precision(dev):
     assert rel_err(got, want) < TOL[torch.bfloat16]
 
 
-def test_long_chunks_take_the_product_path(dev):
-    """chunks long enough for the batched-product path on the GPU, in a portion that starts and ends inside a chunk"""
-    cfg = O.config([O.attn_layer(heads=4, kv_heads=2, dim=16, vdim=24, chunk=128, dims=8, ff=32),
-                    O.attn_layer(heads=4, kv_heads=2, dim=16, vdim=24, chunk=128, dims=8, kv_from=0)], width=32)
+@pytest.mark.parametrize("chunk,sizes", [(128, [50, 390, 10]), (300, [140, 310]), (300, [5, 445])])
+def test_long_chunks_take_the_product_path(dev, chunk, sizes):
+    """pieces of chunks long enough for the batched-product path on the GPU: whole chunks inside a portion that
+    starts and ends mid-chunk, the start of a chunk, and the rest of a chunk whose first keys an earlier step left"""
+    cfg = O.config([O.attn_layer(heads=4, kv_heads=2, dim=16, vdim=24, chunk=chunk, dims=8, ff=32),
+                    O.attn_layer(heads=4, kv_heads=2, dim=16, vdim=24, chunk=chunk, dims=8, kv_from=0)], width=32)
     W = O.random_weights(cfg, 15)
     toks = O.random_tokens(cfg, 450, 15)
     want = O.forward(cfg, W, toks)
     for dtype in (torch.float32, torch.bfloat16):
-        got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", 50)], [("a", 390)], [("a", 10)]])["a"]
+        got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", n)] for n in sizes])["a"]
         assert rel_err(got, want) < TOL[dtype]
 
 
