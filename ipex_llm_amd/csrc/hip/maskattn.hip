@@ -153,6 +153,10 @@ __device__ __forceinline__ int64_t first_key(int64_t p, int mask, int size) {
   return 0;
 }
 
+template <typename E> struct Chunk4;
+template <> struct Chunk4<float> { typedef uint4 type; };
+template <> struct Chunk4<__bf16> { typedef uint2 type; };
+
 // LDS: qs f32 [HB][DQ] | per wave: tile E [KT][DP] (key d | value dv), weights f32 [HB][KT]
 template <typename E, int RC, int HB>
 __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q, const E* __restrict__ rows, int bs,
@@ -162,6 +166,7 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
                                                     E* __restrict__ out, float* __restrict__ part, int H, int G, int d,
                                                     int dv, int DQ, int DP) {
   extern __shared__ __align__(16) unsigned char smem[];
+  typedef typename Chunk4<E>::type C4;
   const int rep = H / G;
   const int nhb = (rep + HB - 1) / HB;                              // head blocks per key head
   const int nsplit = gridDim.z, zs = blockIdx.z;
@@ -201,10 +206,33 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
     const int64_t k0 = (int64_t)ti * KT;
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
-    for (int i = lane; i < nvalid * D; i += 64) {
-      const int j = i / D, c = i - j * D;
-      const E* src = rows + (row0 + j) * RW + (c < d ? (int64_t)g * d + c : (int64_t)G * d + (int64_t)g * dv + (c - d));
-      kt[j * DP + (c < d ? c : DQ + (c - d))] = *src;
+    if (((d | dv) & 3) == 0) {
+      // 4-element chunks (the key part, then the value part of every row), four requests in flight per lane
+      const int cd = d >> 2, cpr = (d + dv) >> 2, n4 = nvalid * cpr;
+      for (int i0 = lane; i0 < n4; i0 += 256) {
+        C4 v[4];
+        int dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int i = i0 + 64 * u;
+          if (i < n4) {
+            const int j = i / cpr, c = i - j * cpr;
+            const E* src = rows + (row0 + j) * RW +
+                           (c < cd ? (int64_t)g * d + 4 * c : (int64_t)G * d + (int64_t)g * dv + 4 * (c - cd));
+            v[u] = *(const C4*)src;
+            dst[u] = j * DP + (c < cd ? 4 * c : DQ + 4 * (c - cd));
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+          if (i0 + 64 * u < n4) *(C4*)(kt + dst[u]) = v[u];
+      }
+    } else {
+      for (int i = lane; i < nvalid * D; i += 64) {
+        const int j = i / D, c = i - j * D;
+        const E* src = rows + (row0 + j) * RW + (c < d ? (int64_t)g * d + c : (int64_t)G * d + (int64_t)g * dv + (c - d));
+        kt[j * DP + (c < d ? c : DQ + (c - d))] = *src;
+      }
     }
     wave_sync();
     float s[HB];

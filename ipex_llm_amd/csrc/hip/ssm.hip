@@ -53,32 +53,72 @@ __device__ __forceinline__ float silu(float z) { return z / (1.0f + expf(-z)); }
 constexpr int kMaxTaps = 16;
 
 // ------------------------------------------------------------------ convolution
-template <typename E>
+// V consecutive channels per thread (V = 4: 4-element accesses; the launcher checks sizes and alignment)
+template <typename E, int V> struct LdV;
+template <typename E> struct LdV<E, 1> {
+  static __device__ __forceinline__ void ld(const E* p, float* v) { v[0] = ldf(p); }
+};
+template <> struct LdV<float, 4> {
+  static __device__ __forceinline__ void ld(const float* p, float* v) {
+    const float4 a = *(const float4*)p;
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+  }
+};
+template <> struct LdV<__bf16, 4> {
+  typedef __bf16 B4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ void ld(const __bf16* p, float* v) {
+    const B4 a = *(const B4*)p;
+    v[0] = (float)a[0], v[1] = (float)a[1], v[2] = (float)a[2], v[3] = (float)a[3];
+  }
+};
+template <int V> __device__ __forceinline__ void stv(float* p, const float* v);
+template <> __device__ __forceinline__ void stv<1>(float* p, const float* v) { p[0] = v[0]; }
+template <> __device__ __forceinline__ void stv<4>(float* p, const float* v) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+template <typename E, int V>
 __global__ void __launch_bounds__(256) conv_silu_k(const E* __restrict__ u, int64_t u_ld, const float* __restrict__ w,
                                                   const float* __restrict__ bias, int taps, float* __restrict__ state,
                                                   const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_of,
                                                   const int32_t* __restrict__ slots, const int64_t* __restrict__ pos,
                                                   float* __restrict__ out, int C, bool single) {
   const int t = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int c = V * (blockIdx.y * blockDim.x + threadIdx.x);
   if (c >= C) return;
   const int b = seq_of[t];
   const int i = t - cu[b];                                          // index inside the portion
   const int64_t p = pos[t];
   float* st = state + (int64_t)slots[b] * (taps - 1) * C + c;       // [taps - 1][C], oldest first
-  float acc = bias[c];
-  float hist[kMaxTaps];                                             // inputs of positions p - taps + 1 .. p
+  float acc[V];
+  LdV<float, V>::ld(bias + c, acc);
   for (int j = 0; j < taps; j++) {
-    const int back = taps - 1 - j;
-    float v = 0.f;
-    if (back <= i) v = ldf(u + (int64_t)(t - back) * u_ld + c);
-    else if (p - back >= 0) v = st[(int64_t)(taps - 1 + i - back) * C];
-    hist[j] = v;
-    acc = fmaf(w[(int64_t)c * taps + j], v, acc);
+    const int back = taps - 1 - j;                                  // the input of position p - back
+    float v[V];
+#pragma unroll
+    for (int q = 0; q < V; q++) v[q] = 0.f;
+    if (back <= i) LdV<E, V>::ld(u + (int64_t)(t - back) * u_ld + c, v);
+    else if (p - back >= 0) LdV<float, V>::ld(st + (int64_t)(taps - 1 + i - back) * C, v);
+#pragma unroll
+    for (int q = 0; q < V; q++) acc[q] = fmaf(w[(int64_t)(c + q) * taps + j], v[q], acc[q]);
   }
-  out[(int64_t)t * C + c] = silu(acc);
-  if (single)                                                       // the only token of its sequence: advance the state
-    for (int j = 1; j < taps; j++) st[(int64_t)(j - 1) * C] = hist[j];
+#pragma unroll
+  for (int q = 0; q < V; q++) acc[q] = silu(acc[q]);
+  stv<V>(out + (int64_t)t * C + c, acc);
+  if (single && taps > 1) {
+    // the only token of its sequence (i == 0): the slot moves up by one position; row j held position
+    // p - (taps - 1 - j), positions before 0 are zero whatever the slot held
+    for (int j = 1; j < taps - 1; j++) {
+      float v[V];
+#pragma unroll
+      for (int q = 0; q < V; q++) v[q] = 0.f;
+      if (p - (taps - 1 - j) >= 0) LdV<float, V>::ld(st + (int64_t)j * C, v);
+      stv<V>(st + (int64_t)(j - 1) * C, v);
+    }
+    float v[V];
+    LdV<E, V>::ld(u + (int64_t)t * u_ld + c, v);
+    stv<V>(st + (int64_t)(taps - 2) * C, v);
+  }
 }
 
 // after a portion of n tokens that started at position p0: the slot holds the inputs of positions p0 + n - taps + 1 ..
@@ -265,16 +305,22 @@ void conv_silu(bool bf16, const void* u, int64_t u_ld, const float* w, const flo
                const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* out, int T,
                int B, int C, bool single, hipStream_t st) {
   if (T <= 0 || C <= 0) return;
-  dim3 grid(T, (C + 255) / 256), gs(B, (C + 255) / 256);
+  const size_t eb = bf16 ? 2 : 4;
+  const bool v4 = (C & 3) == 0 && (u_ld & 3) == 0 && ((uintptr_t)u % (4 * eb)) == 0;
+  const int cw = v4 ? C / 4 : C;
+  dim3 grid(T, (cw + 255) / 256), gs(B, (C + 255) / 256);
+#define SSM_CONV(E, V)                                                                                               \
+  conv_silu_k<E, V><<<grid, 256, 0, st>>>((const E*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C, single)
   if (bf16) {
-    conv_silu_k<__bf16><<<grid, 256, 0, st>>>((const __bf16*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C,
-                                              single);
+    if (v4) SSM_CONV(__bf16, 4);
+    else SSM_CONV(__bf16, 1);
     if (!single && taps > 1) conv_state_k<__bf16><<<gs, 256, 0, st>>>((const __bf16*)u, u_ld, taps, state, cu, slots, pos, C);
   } else {
-    conv_silu_k<float><<<grid, 256, 0, st>>>((const float*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C,
-                                             single);
+    if (v4) SSM_CONV(float, 4);
+    else SSM_CONV(float, 1);
     if (!single && taps > 1) conv_state_k<float><<<gs, 256, 0, st>>>((const float*)u, u_ld, taps, state, cu, slots, pos, C);
   }
+#undef SSM_CONV
 }
 
 void selective_scan(bool bf16, const float* x, int64_t x_ld, const float* Bm, int64_t b_ld, const float* Cm,

@@ -135,17 +135,18 @@ def test_add_norm_and_gates(dev):
             assert (got.double().cpu() - ref).abs().max() < (1e-5 if act == torch.float32 else 5e-2)
 
 
+@pytest.mark.parametrize("C,off", [(37, 2), (40, 4)])
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
-def test_convolution_state(dev, taps):
+def test_convolution_state(dev, taps, C, off):
     """portions of every length from the start of a sequence and from its middle, sequences side by side,
     slots that held other sequences before"""
     from ipex_llm_amd.ops import ssm as SSM
     g = torch.Generator().manual_seed(taps)
-    C, n = 37, 23
+    n = 23                                                          # (C, off): channels one by one / four at a time
     w = torch.randn(C, taps, generator=g)
     b = torch.randn(C, generator=g)
-    seqs = [torch.randn(n, C + 5, generator=g) for _ in range(3)]
-    want = [O.silu(O.causal_conv(u[:, 2:2 + C].double(), w.double(), b.double())) for u in seqs]
+    seqs = [torch.randn(n, C + 8, generator=g) for _ in range(3)]
+    want = [O.silu(O.causal_conv(u[:, off:off + C].double(), w.double(), b.double())) for u in seqs]
     state = torch.randn(5, taps - 1, C, generator=g).to(dev)            # rubbish of earlier owners
     cuts = [[1, 1, 1, 2, 3, 5, 10], [23], [2, 1, 1, 19]]
     at = [0, 0, 0]
@@ -156,7 +157,7 @@ def test_convolution_state(dev, taps):
         starts = [at[s] for s in act]
         cu, seq_of, _, pos = ragged(lens, starts, dev)
         slots = torch.tensor([s + 1 for s in act], dtype=torch.int32, device=dev)
-        u = torch.cat([seqs[s][at[s]:at[s] + m] for s, m in zip(act, lens)]).to(dev)[:, 2:2 + C]
+        u = torch.cat([seqs[s][at[s]:at[s] + m] for s, m in zip(act, lens)]).to(dev)[:, off:off + C]
         out = SSM.conv_silu(u, w.to(dev), b.to(dev), state, cu, seq_of, slots, pos, lens)
         o = 0
         for s, m in zip(act, lens):
