@@ -41,6 +41,21 @@ Building blocks (each usable by any design that lists it in its layer specs):
   values of an earlier layer (``kv_from``) instead of its own.
 * ``LatentAttention`` also takes a sliding window, the half-split rotary layout
   (folded into the weights' row order) and an element-wise output gate.
+* ``MaskedAttention`` also takes short causal convolutions on q / k / v right
+  after the projection (their last inputs are state), a tanh cap on the
+  scores, a sink of a fixed score, a window that keeps the sequence's first
+  tokens visible, an [H, H] mixing of the heads' weights *after* the softmax,
+  a sigmoid output gate, and the wavelength rule of Llama 3.1 for its rotary
+  frequencies.
+* ``MinGRU``            minGRU: gates that read only the current token,
+  S' = (1 - z) S + z c element by element over f32 state, SiLU output gate.
+* ``GatedLinearAttention``  per head S' = diag(alpha) S + k v^T, o = S'^T q with
+  a decay per key channel alpha = sigmoid(low-rank(h))^(1 / tau), per-head RMS
+  norm and a SiLU output gate; f32 state.
+* ``SideBySide``        two mixers on the same input (one fused projection),
+  each result RMS-normed over the width, then their mean.
+* ``SoftmaxMoE``        experts whose weights are the softmax over the chosen
+  router logits and multiply the experts' *outputs*; SiLU-gated experts.
 
 Block layouts.  ``pre_norm`` (``PreNormLayer``): x += mixer(norm1(x)),
 x += ff(norm2(x)) with vector RMS norms; each sublayer's result is added by
@@ -51,6 +66,10 @@ x += mult * LN(mixer(x)), x += mult * LN(ff(x)).  ``parallel``
 are summed and added: h = norm(x), x += ls1 * mixer(h + conv(h)) + ls2 * ff(h),
 with an optional short causal convolution in front of the mixer (its last
 inputs are per-sequence state) and an optional token-side input afterwards.
+``parallel2`` (``TwoNormParallelLayer``): two LayerNorms of the same x, the
+mixer's input shifted towards the previous token's:
+h = LN1(x), x += mixer(h + (h_prev - h) * mu) + ff(LN2(x)), then the token-side
+input.
 The residual stream is f32 throughout; projections run in the model's
 activation dtype through the vendor GEMM, everything else in the kernels of
 ``ops/seqmix.py`` and ``ops/blockmix.py``.
@@ -69,6 +88,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from ..ops import blockmix as BM
+from ..ops import gatedmix as GM
 from ..ops import maskattn as MA
 from ..ops import seqmix as SM
 from ..ops import ssm as SSM
@@ -80,7 +100,7 @@ from .decoder import AttnMeta
 class RotarySpec:
     dims: int
     base: float = 10000.0
-    scaling: Optional[dict] = None          # YaRN: factor, original, fast, slow
+    scaling: Optional[dict] = None          # YaRN: factor, original, fast, slow | Llama 3.1: factor, low, high, original
     layout: Optional[str] = None            # "pairs" (2i, 2i+1) | "half" (i, i + dims/2); None: the mixer's own
 
 
@@ -88,6 +108,7 @@ class RotarySpec:
 class MaskSpec:
     kind: str = "causal"                    # "causal" | "window" (itself and size - 1 before) | "chunk" (aligned blocks)
     size: int = 0
+    keep_first: int = 0                     # window: the sequence's first keep_first tokens stay visible as well
 
 
 @dataclass
@@ -127,6 +148,33 @@ class MaskedAttentionSpec:
     bias: bool = True                       # q / k / v projections carry biases
     sink: bool = True                       # a learned number per head in the softmax's denominator
     kv_from: Optional[int] = None           # read this layer's cache rows instead of projecting keys and values
+    taps: int = 0                           # >= 1: causal per-channel convolutions on q / k / v right after the projection
+    softcap: float = 0.0                    # > 0: score <- softcap tanh(score / softcap)
+    sink_score: Optional[float] = None      # a sink of this fixed score (no tensor) instead of a learned one
+    talk: bool = False                      # [H, H] mixing of the heads' weights after the softmax
+    out_gate: bool = False                  # element-wise sigmoid gate on the joined heads
+
+
+@dataclass
+class MinGRUSpec:
+    width: int
+
+
+@dataclass
+class GatedLinearAttentionSpec:
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    rank: int                               # of the low-rank decay projection
+
+
+@dataclass
+class SideBySideSpec:
+    left: object                            # (kind, spec) pairs of MIXERS
+    right: object
+    left_kind: str = "masked_attention"
+    right_kind: str = "gated_linear_attention"
 
 
 @dataclass
@@ -163,7 +211,7 @@ class ReluSqFFSpec:
 @dataclass
 class ExpertSpec:
     ff: int
-    limit: float
+    limit: float = float("inf")
     alpha: float = 1.702
 
 
@@ -200,15 +248,21 @@ class HybridSpec:
     bigram: Optional[BigramSpec] = None
     final_softcap: float = 0.0              # read by the engines' shared helpers
     logit_scale: float = 1.0                # the logits are multiplied by it
-    block: str = "post_norm"                # "post_norm" | "parallel" | "pre_norm"
+    block: str = "post_norm"                # "post_norm" | "parallel" | "parallel2" | "pre_norm"
     norm: str = "layer_norm"                # "layer_norm" | "rms_scalar" (one number) | "rms" (a vector)
     layer_scale: bool = False               # parallel blocks: per-coordinate scales on both sublayers' results
     canon_taps: int = 0                     # parallel blocks: taps of the convolution in front of the mixer (0: none)
     side_dim: int = 0                       # per-layer slice of the token-side table (0: none)
+    tied_head: bool = False                 # the logits are products with the embedding table
 
     @property
     def num_layers(self) -> int:
         return len(self.layers)
+
+
+def _spec_list(c) -> list:
+    """a mixer's cache request (one entry, a list of entries or None) as a list"""
+    return list(c) if isinstance(c, list) else [c]
 
 
 # ---------------------------------------------------------------------- mixers
@@ -373,32 +427,53 @@ class SSMMixer(nn.Module):
 
 class MaskedAttention(nn.Module):
     """``w_q`` [H d, W], ``w_k`` [G d, W], ``w_v`` [G dv, W] (``w_k`` / ``w_v`` None with ``kv_from``), biases or
-    None, norm weights per ``qk_norm``, ``sink`` [H] or None, ``w_o`` [W, H dv]."""
+    None, norm weights per ``qk_norm``, ``sink`` [H] or None, ``w_o`` [W, H dv]; optional ``conv`` = (q, k, v)
+    weights [channels, taps] (k / v None with ``kv_from``), ``talk`` [H, H], ``w_g`` [H dv, W]."""
     cache_kind = "rows"
 
-    def __init__(self, s: MaskedAttentionSpec, w_q, w_k, w_v, b_q, b_k, b_v, q_norm, k_norm, sink, w_o):
+    def __init__(self, s: MaskedAttentionSpec, w_q, w_k, w_v, b_q, b_k, b_v, q_norm, k_norm, sink, w_o, conv=None,
+                 talk=None, w_g=None):
         super().__init__()
         if s.heads % s.kv_heads:
             raise ValueError("heads must be a multiple of kv_heads")
         if s.mask is None or s.mask.kind not in MA.MASKS or (s.mask.kind != "causal" and s.mask.size < 1):
             raise ValueError("mask: causal, or window / chunk with a size of at least 1")
+        if s.mask.keep_first and s.mask.kind != "window":
+            raise ValueError("keep_first belongs to a window")
         if s.qk_norm not in ("none", "head", "whole"):
             raise ValueError(f"unknown qk_norm {s.qk_norm!r}")
         self.s = s
         shared = s.kv_from is not None
-        self.w_in = nn.Parameter((w_q if shared else torch.cat([w_q, w_k, w_v], 0)).contiguous(), requires_grad=False)
+        parts = [w_q] if shared else [w_q, w_k, w_v]
+        self.n_qkv = sum(int(w.shape[0]) for w in parts)
+        if s.out_gate:
+            parts = parts + [w_g]
+        self.w_in = nn.Parameter(torch.cat(parts, 0).contiguous(), requires_grad=False)
         self.b_in = None
         if s.bias:
-            self.b_in = nn.Parameter((b_q if shared else torch.cat([b_q, b_k, b_v], 0)).contiguous(), requires_grad=False)
+            bs = [b_q] if shared else [b_q, b_k, b_v]
+            if s.out_gate:
+                bs = bs + [torch.zeros(w_g.shape[0], dtype=b_q.dtype, device=b_q.device)]
+            self.b_in = nn.Parameter(torch.cat(bs, 0).contiguous(), requires_grad=False)
+        self.conv = None
+        if s.taps >= 1:
+            cw = [conv[0]] if shared else list(conv)
+            self.conv = nn.Parameter(torch.cat(cw, 0).float().contiguous(), requires_grad=False)      # [q | k | v] channels
         self.q_norm = nn.Parameter(q_norm, requires_grad=False) if q_norm is not None else None
         self.k_norm = nn.Parameter(k_norm, requires_grad=False) if k_norm is not None else None
+        if s.sink_score is not None:
+            sink = torch.full((s.heads,), float(s.sink_score), device=w_o.device)
         self.sink = nn.Parameter(sink.float().contiguous(), requires_grad=False) if sink is not None else None
+        self.talk = nn.Parameter(talk.float().contiguous(), requires_grad=False) if s.talk else None
         self.w_o = nn.Parameter(w_o, requires_grad=False)
         self.table: Optional[torch.Tensor] = None
 
     def cache_spec(self):
         s = self.s
-        return None if s.kv_from is not None else ("rows", s.kv_heads * (s.dim + s.vdim))
+        out = [] if s.kv_from is not None else [("rows", s.kv_heads * (s.dim + s.vdim))]
+        if self.conv is not None:
+            out.append(("state", {"conv": (s.taps - 1, self.n_qkv)}))
+        return out[0] if len(out) == 1 else (out or None)
 
     def ensure_table(self, max_pos: int):
         if self.s.rot is None or self.s.rot.dims == 0:
@@ -409,24 +484,150 @@ class MaskedAttention(nn.Module):
         return self.table
 
     def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        return self.mix(BM.linear(xa, self.w_in, self.b_in), pos, slots, meta, cache, li, eps)
+
+    def mix(self, y, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        """``y``: this mixer's columns of the input projection, ``[q | k | v | gate]``"""
         s = self.s
-        T, H, G, d, dv = xa.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
-        y = BM.linear(xa, self.w_in, self.b_in)
+        T, H, G, d, dv = y.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        gate = y[:, self.n_qkv:] if s.out_gate else None
+        if self.conv is not None:
+            y = GM.causal_conv(y[:, :self.n_qkv], self.conv, cache.state[li]["conv"], meta.cu_q, meta.seq_of,
+                               meta.state_slots, pos, meta.q_lens_host)
         q = y[:, :H * d].view(T, H, d)
         layout = (s.rot.layout if s.rot is not None else None) or "half"
+        table = self.table if s.rot is not None and s.rot.dims else None
         if s.kv_from is None:
             k = y[:, H * d:(H + G) * d].view(T, G, d)
-            v = y[:, (H + G) * d:].view(T, G, dv)
+            v = y[:, (H + G) * d:(H + G) * d + G * dv].view(T, G, dv)
             rows = cache.rows[li]
-            qf = MA.qkv_norm_rope_store(q, k, v, self.q_norm, self.k_norm, s.qk_norm == "whole", eps, self.table,
+            qf = MA.qkv_norm_rope_store(q, k, v, self.q_norm, self.k_norm, s.qk_norm == "whole", eps, table,
                                         layout, pos, slots, rows)
         else:
             rows = cache.rows[s.kv_from]
-            qf = MA.qkv_norm_rope_store(q, None, None, self.q_norm, None, s.qk_norm == "whole", eps, self.table,
+            qf = MA.qkv_norm_rope_store(q, None, None, self.q_norm, None, s.qk_norm == "whole", eps, table,
                                         layout, pos, slots, None)
         o = MA.masked_attention(qf, rows, G, dv, meta.block_tables, meta.seq_of, pos, s.scale, s.mask.kind, s.mask.size,
-                                self.sink, meta.q_lens_host, meta.seq_lens_host, xa.dtype)
+                                self.sink, meta.q_lens_host, meta.seq_lens_host, y.dtype, softcap=s.softcap,
+                                keep_first=s.mask.keep_first, talk=self.talk)
+        if gate is not None:
+            o = MA.sigmoid_gate(o, gate)
         return BM.linear(o, self.w_o)
+
+
+class MinGRU(nn.Module):
+    """``w_z`` / ``w_x`` / ``w_g`` [width, W], ``b_z`` / ``b_x`` [width], ``w_o`` [W, width]: z = sigmoid(W_z h + b_z),
+    u = W_x h + b_x, candidate u + 1/2 (u >= 0) or sigmoid(u) (u < 0), S' = (1 - z) S + z c, W_o (S' silu(W_g h))."""
+    cache_kind = "state"
+
+    def __init__(self, s: MinGRUSpec, w_z, w_x, w_g, b_z, b_x, w_o):
+        super().__init__()
+        self.s = s
+        self.w_in = nn.Parameter(torch.cat([w_z, w_x, w_g], 0).contiguous(), requires_grad=False)
+        self.b_in = nn.Parameter(torch.cat([b_z, b_x, torch.zeros_like(b_x)], 0).contiguous(), requires_grad=False)
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+
+    def cache_spec(self):
+        return ("state", {"gru": (self.s.width,)})
+
+    def ensure_table(self, max_pos: int):
+        return None
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        return self.mix(BM.linear(xa, self.w_in, self.b_in), pos, slots, meta, cache, li, eps)
+
+    def mix(self, y, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        o = GM.mingru_scan(y, self.s.width, cache.state[li]["gru"], meta.cu_q, meta.state_slots, pos, meta.q_lens_host)
+        return BM.linear(o, self.w_o)
+
+
+class GatedLinearAttention(nn.Module):
+    """``w_q`` / ``w_k`` [H d, W], ``w_v`` / ``w_g`` [H dv, W], ``w_a1`` [rank, W], ``w_a2`` [H d, rank] with bias
+    ``b_a2``, ``norm`` [dv], ``w_o`` [W, H dv]."""
+    cache_kind = "state"
+
+    def __init__(self, s: GatedLinearAttentionSpec, w_q, w_k, w_v, w_g, w_a1, w_a2, b_a2, norm, w_o):
+        super().__init__()
+        if s.tau <= 0:
+            raise ValueError("tau must be positive")
+        self.s = s
+        self.w_in = nn.Parameter(torch.cat([w_q, w_k, w_v, w_g, w_a1], 0).contiguous(), requires_grad=False)
+        self.b_in = None
+        self.w_a2 = nn.Parameter(w_a2, requires_grad=False)
+        self.b_a2 = nn.Parameter(b_a2, requires_grad=False)
+        self.norm = nn.Parameter(norm, requires_grad=False)
+        self.w_o = nn.Parameter(w_o, requires_grad=False)
+
+    def cache_spec(self):
+        s = self.s
+        return ("state", {"gla": (s.heads, s.dim, s.vdim)})
+
+    def ensure_table(self, max_pos: int):
+        return None
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        return self.mix(BM.linear(xa, self.w_in), pos, slots, meta, cache, li, eps)
+
+    def mix(self, y, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        s = self.s
+        T, H, d, dv = y.shape[0], s.heads, s.dim, s.vdim
+        nqk, nv = H * d, H * dv
+        q, k = y[:, :nqk].view(T, H, d), y[:, nqk:2 * nqk].view(T, H, d)
+        v = y[:, 2 * nqk:2 * nqk + nv].view(T, H, dv)
+        g = y[:, 2 * nqk + nv:2 * nqk + 2 * nv]
+        a = BM.linear(y[:, 2 * nqk + 2 * nv:].contiguous(), self.w_a2, self.b_a2).view(T, H, d)
+        o = GM.gla_scan(q, k, v, a, s.tau, d ** -0.5, cache.state[li]["gla"], meta.cu_q, meta.state_slots, pos,
+                        meta.q_lens_host)
+        return BM.linear(GM.head_rms_silu(o, self.norm, g, eps, y.dtype), self.w_o)
+
+
+class SideBySide(nn.Module):
+    """Two mixers reading the same input: one projection launch over both mixers' input rows, then
+    ``(rms_norm(left) * out_l + rms_norm(right) * out_r) / 2`` over the model width."""
+    cache_kind = "both"
+
+    def __init__(self, left: nn.Module, right: nn.Module, out_l, out_r):
+        super().__init__()
+        self.left, self.right = left, right
+        ws, bs = [left.w_in, right.w_in], [left.b_in, right.b_in]
+        self.n_left = int(left.w_in.shape[0])
+        self.w_in = nn.Parameter(torch.cat([w.data for w in ws], 0).contiguous(), requires_grad=False)
+        self.b_in = None
+        if any(b is not None for b in bs):
+            bs = [b.data if b is not None else torch.zeros(w.shape[0], dtype=w.dtype, device=w.device)
+                  for w, b in zip(ws, bs)]
+            self.b_in = nn.Parameter(torch.cat(bs, 0).contiguous(), requires_grad=False)
+        left.w_in = right.w_in = None                  # the fused copy is the one that runs
+        left.b_in = right.b_in = None
+        self.out_l = nn.Parameter(out_l, requires_grad=False)
+        self.out_r = nn.Parameter(out_r, requires_grad=False)
+
+    def cache_spec(self):
+        out = []
+        for m in (self.left, self.right):
+            c = m.cache_spec()
+            out += c if isinstance(c, list) else ([c] if c is not None else [])
+        return out
+
+    def ensure_table(self, max_pos: int):
+        self.left.ensure_table(max_pos)
+        self.right.ensure_table(max_pos)
+
+    @property
+    def table(self):
+        return getattr(self.left, "table", None)
+
+    @table.setter
+    def table(self, v):
+        for m in (self.left, self.right):
+            if hasattr(m, "table"):
+                m.table = v
+
+    def forward(self, xa, pos, slots, meta: AttnMeta, cache, li: int, eps: float):
+        y = BM.linear(xa, self.w_in, self.b_in)
+        a = self.left.mix(y[:, :self.n_left], pos, slots, meta, cache, li, eps)
+        b = self.right.mix(y[:, self.n_left:], pos, slots, meta, cache, li, eps)
+        return GM.rms_pair_mean(a, b, self.out_l, self.out_r, eps, xa.dtype)
 
 
 class GroupedAttention(nn.Module):
@@ -503,6 +704,25 @@ class SigmoidMoE(nn.Module):
         return y, ys
 
 
+class SoftmaxMoE(nn.Module):
+    """``w_gu`` [E, 2 ff, W] (every expert's gate rows, then its up rows), ``w_down`` [E, W, ff].  The router's
+    logits are f32 products with the input; the ``top`` largest win, their weights are the softmax over the chosen
+    logits only and multiply the experts' *outputs*; experts ``W_down (silu(W_gate h) * (W_up h))``."""
+
+    def __init__(self, s: MoESpec, router, w_gu, w_down):
+        super().__init__()
+        self.s = s
+        self.router = nn.Parameter(router.float().contiguous(), requires_grad=False)
+        self.w_gu = nn.Parameter(w_gu.contiguous(), requires_grad=False)
+        self.w_down = nn.Parameter(w_down.contiguous(), requires_grad=False)
+
+    def forward(self, xa, x32=None):
+        s = self.s
+        idx, wts = BM.moe_route(F.linear(xa.float() if x32 is None else x32, self.router), s.top, "softmax")
+        y = BM.moe_experts(xa, idx, wts, self.w_gu, self.w_down, float("inf"), 1.0, 0.0, "output")
+        return y, None
+
+
 class TokenSide(nn.Module):
     """x += rms_norm(W_proj (gelu_tanh(W_gate x) * e)) * w, with e the layer's
     slice of the token-side table's row of the token."""
@@ -527,7 +747,7 @@ class HybridLayer(nn.Module):
         self.norm2 = nn.Parameter(norm2, requires_grad=False) if norm2 is not None else None
 
     def cache_specs(self):
-        return [self.mixer.cache_spec()]
+        return _spec_list(self.mixer.cache_spec())
 
     def forward(self, x, xa, ids, pos, slots, meta, cache, li: int, model):
         s, act = model.spec, model.dtype
@@ -550,7 +770,7 @@ class PreNormLayer(nn.Module):
         self.norm2 = nn.Parameter(norm2, requires_grad=False) if norm2 is not None else None
 
     def cache_specs(self):
-        return [self.mixer.cache_spec()]
+        return _spec_list(self.mixer.cache_spec())
 
     def forward(self, x, carry, ids, pos, slots, meta, cache, li: int, model):
         s, act = model.spec, model.dtype
@@ -577,7 +797,7 @@ class ParallelLayer(nn.Module):
         self.ls2 = nn.Parameter(ls2.float(), requires_grad=False) if ls2 is not None else None
 
     def cache_specs(self):
-        out = [self.mixer.cache_spec()]
+        out = _spec_list(self.mixer.cache_spec())
         if self.canon is not None and self.canon.shape[1] > 1:
             out.append(("state", {"canon": (self.canon.shape[1] - 1, self.canon.shape[0])}))
         return out
@@ -598,11 +818,47 @@ class ParallelLayer(nn.Module):
         return xa
 
 
+class TwoNormParallelLayer(nn.Module):
+    """h = LN1(x) shifted towards the previous token's (``shift`` [W] or None), x += mixer(h) + ff(LN2(x)); then the
+    token-side input.  LayerNorms with a weight and no bias; the previous token's LN1(x) is per-sequence state.
+    ``mlp`` returns (result, second result or None) and may be None."""
+
+    def __init__(self, mixer: nn.Module, norm1: torch.Tensor, mlp: Optional[nn.Module], norm2: Optional[torch.Tensor],
+                 shift: Optional[torch.Tensor] = None, side: Optional[TokenSide] = None):
+        super().__init__()
+        self.mixer, self.mlp, self.side = mixer, mlp, side
+        self.norm1 = nn.Parameter(norm1, requires_grad=False)
+        self.norm2 = nn.Parameter(norm2, requires_grad=False) if norm2 is not None else None
+        self.shift = nn.Parameter(shift.float().contiguous(), requires_grad=False) if shift is not None else None
+
+    def cache_specs(self):
+        out = _spec_list(self.mixer.cache_spec())
+        if self.shift is not None:
+            out.append(("state", {"shift": (self.norm1.shape[0],)}))
+        return out
+
+    def forward(self, x, xa, ids, pos, slots, meta, cache, li: int, model):
+        s, act = model.spec, model.dtype
+        st = cache.state[li]["shift"] if self.shift is not None else None
+        h1, h2 = GM.layer_norm_pair_shift(x, self.norm1, self.norm2 if self.mlp is not None else None, self.shift,
+                                          s.norm_eps, st, meta.cu_q, meta.seq_of, meta.state_slots, pos,
+                                          meta.q_lens_host, act)
+        ym = self.mixer(h1, pos, slots, meta, cache, li, s.norm_eps)
+        y2, y3 = self.mlp(h2, None) if self.mlp is not None else (None, None)
+        xa = BM.residual_add_scaled_(x, ym, None, y2, y3, None, act)
+        if self.side is not None:
+            xa = self.side(x, xa, ids, model.side_embed, s.norm_eps, act)
+        return xa
+
+
 # name -> (spec class, module class): a design's config reader maps its layer
 # types onto these
 MIXERS: Dict[str, tuple] = {"latent_attention": (LatentAttentionSpec, LatentAttention), "mlstm": (MLSTMSpec, MLSTM),
                             "grouped_attention": (GroupedAttentionSpec, GroupedAttention),
-                            "ssm": (SSMSpec, SSMMixer), "masked_attention": (MaskedAttentionSpec, MaskedAttention)}
+                            "ssm": (SSMSpec, SSMMixer), "masked_attention": (MaskedAttentionSpec, MaskedAttention),
+                            "mingru": (MinGRUSpec, MinGRU),
+                            "gated_linear_attention": (GatedLinearAttentionSpec, GatedLinearAttention),
+                            "side_by_side": (SideBySideSpec, SideBySide)}
 
 
 # ---------------------------------------------------------------------- model
@@ -620,7 +876,8 @@ class HybridCausalLM(nn.Module):
         self.side_embed = nn.Parameter(side_embed, requires_grad=False) if side_embed is not None else None
         self.layers = nn.ModuleList(layers)
         self.norm = nn.Parameter(final_norm, requires_grad=False)
-        self.lm_head = nn.Parameter(head, requires_grad=False)
+        # a tied head (head None) is the embedding table itself
+        self.lm_head = nn.Parameter(head, requires_grad=False) if head is not None else self.embed_tokens
         self.tp_group = None
         self.first_stage = self.last_stage = True
         self.capture_layers: Optional[list] = None      # debugging: residual stream after every layer
@@ -709,4 +966,6 @@ class HybridCausalLM(nn.Module):
         if return_hidden:
             return xn
         logits = BM.linear(xn, self.lm_head).float()
+        if s.final_softcap:
+            return GM.softcap_(logits, s.final_softcap)
         return logits.mul_(s.logit_scale) if s.logit_scale != 1.0 else logits

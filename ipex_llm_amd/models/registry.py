@@ -19,6 +19,7 @@ NATIVE_ARCHITECTURES = {
     "Zamelix": "ipex_llm_amd.models.zamelix",
     "Masezen": "ipex_llm_amd.models.masezen",
     "Vogolix": "ipex_llm_amd.models.vogolix",
+    "Zoguzen": "ipex_llm_amd.models.zoguzen",
 }
 
 

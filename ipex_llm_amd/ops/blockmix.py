@@ -31,6 +31,9 @@ def _ops():
     return torch.ops.ipex_llm_amd
 
 
+ROUTE_MODES = {"sigmoid": 0, "softmax": 1}
+
+
 # ------------------------------------------------------------------ projections
 def linear(x: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x W^T (+ b)`` for rows ``x`` [T, K] and ``w`` [N, K]: decode-size steps (at most 16 rows, 16-bit) stream
@@ -337,36 +340,50 @@ def side_gate(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, offset: i
 
 
 # ------------------------------------------------------------------ experts
-def moe_route(z: torch.Tensor, top: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def moe_route(z: torch.Tensor, top: int, mode: str = "sigmoid") -> Tuple[torch.Tensor, torch.Tensor]:
     """Router logits ``z`` f32 [T, E] -> the ``top`` experts with the largest
-    ``sigmoid(z)`` per token (int32 [T, top], lowest index first among equals)
-    and those scores themselves as weights (f32 [T, top], not renormalised)."""
+    logits per token (int32 [T, top], lowest index first among equals) and
+    their weights (f32 [T, top]): ``mode`` "sigmoid": ``sigmoid(z)`` of each
+    chosen expert, not renormalised; "softmax": the softmax over the chosen
+    logits only."""
+    if mode not in ROUTE_MODES:
+        raise ValueError(f"unknown router mode {mode!r}")
     if native(z):
-        return _ops().bm_moe_route(z.contiguous(), top)
-    s = torch.sigmoid(z.float())
-    val, idx = torch.sort(s, dim=-1, descending=True, stable=True)
-    return idx[:, :top].to(torch.int32).contiguous(), val[:, :top].contiguous()
+        return _ops().bm_moe_route(z.contiguous(), top, ROUTE_MODES[mode])
+    val, idx = torch.sort(z.float(), dim=-1, descending=True, stable=True)
+    val = val[:, :top]
+    w = torch.sigmoid(val) if mode == "sigmoid" else torch.softmax(val, -1)
+    return idx[:, :top].to(torch.int32).contiguous(), w.contiguous()
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor,
-                limit: float, alpha: float = 1.702) -> torch.Tensor:
-    """Sum over a token's chosen experts of ``expert_e(w h)``: the routing
-    weight multiplies the expert's *input*.  ``h`` [T, W] in the activation
-    dtype, ``w_gu`` [E, 2 ff, W] (gate rows, then up rows), ``w_down`` [E, W, ff];
-    expert: ``W_down (g sigmoid(alpha g) (u + 1))`` with the clamps of
-    ``glu_clamp``.  Returns f32 [T, W]."""
+                limit: float, alpha: float = 1.702, up_shift: float = 1.0, weigh: str = "input") -> torch.Tensor:
+    """Sum over a token's chosen experts.  ``weigh`` "input": ``expert_e(w h)``,
+    the routing weight multiplies the expert's *input*; "output":
+    ``w expert_e(h)``.  ``h`` [T, W] in the activation dtype, ``w_gu``
+    [E, 2 ff, W] (gate rows, then up rows), ``w_down`` [E, W, ff]; expert:
+    ``W_down (g sigmoid(alpha g) (u + up_shift))`` with g = min(gate, limit),
+    u = clamp(up, -limit, limit) (``limit`` may be infinite; alpha = 1,
+    up_shift = 0: the SiLU-gated unit).  Returns f32 [T, W]."""
     T, W = h.shape
     top = idx.shape[1]
+    if weigh not in ("input", "output"):
+        raise ValueError(f"unknown weighing {weigh!r}")
     if native(h):
-        return _ops().bm_moe_experts(h.contiguous(), idx, wts, w_gu, w_down, limit, alpha)
+        return _ops().bm_moe_experts(h.contiguous(), idx, wts, w_gu, w_down, limit, alpha, up_shift, weigh == "output")
     out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
     E = w_gu.shape[0]
+    I = w_gu.shape[1] // 2
     for k in range(top):
-        xin = (h.float() * wts[:, k:k + 1]).to(h.dtype)
+        xin = (h.float() * wts[:, k:k + 1]).to(h.dtype) if weigh == "input" else h
         for e in range(E):
             sel = (idx[:, k] == e).nonzero().squeeze(-1)
             if sel.numel() == 0:
                 continue
-            y = glu_clamp(F.linear(xin[sel], w_gu[e]), limit, alpha)
-            out[sel] += F.linear(y, w_down[e]).float()
+            gu = F.linear(xin[sel], w_gu[e])
+            g = gu[..., :I].float().clamp(max=limit)
+            u = gu[..., I:].float().clamp(-limit, limit)
+            y = (g * torch.sigmoid(alpha * g) * (u + up_shift)).to(h.dtype)
+            r = F.linear(y, w_down[e]).float()
+            out[sel] += r * wts[sel, k:k + 1] if weigh == "output" else r
     return out

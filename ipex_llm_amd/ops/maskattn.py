@@ -112,22 +112,25 @@ GEMM_MIN_CHUNK = int(os.environ.get("ILLM_MASKATTN_GEMM_MIN", "128"))
 def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block_tables: torch.Tensor,
                      seq_of: torch.Tensor, pos: torch.Tensor, scale: float, mask: str, size: int,
                      sink: Optional[torch.Tensor], q_lens: List[int], ctx_lens: List[int],
-                     out_dtype: torch.dtype) -> torch.Tensor:
+                     out_dtype: torch.dtype, softcap: float = 0.0, keep_first: int = 0,
+                     talk: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Grouped-query attention over paged rows ``[keys (G d) | values (G dv)]``.
     For token t (position p), query head h (key / value head h // (H / G)) and
-    the visible keys ``first_visible(p) <= j <= p``:
+    the visible keys ``first_visible(p) <= j <= p`` (and, with ``keep_first``,
+    the keys ``j < keep_first`` of the sequence's start as well):
 
-        s_j = (q[t, h] . key_j) * scale
+        s_j = (q[t, h] . key_j) * scale;   softcap > 0:  s_j <- softcap tanh(s_j / softcap)
         w_j = exp(s_j) / (sum_visible exp(s_i) + exp(sink[h]))      (no sink: the plain softmax)
+        talk [H, H] given:  w_j[h] <- sum_g talk[h, g] w_j[g]       (the heads' weights mixed after the softmax)
         out[t, h] = sum_j w_j value_j
 
     The sink is one more term of the denominator: it has no key and no value,
-    is not scaled and counts once.  ``q`` f32 [T, H, d]; everything is f32.
-    Returns [T, H dv] in ``out_dtype``."""
+    is not scaled or capped, counts once and is not mixed.  ``q`` f32 [T, H, d];
+    everything is f32.  Returns [T, H dv] in ``out_dtype``."""
     T, H, d = q.shape
     if native(q):
         return _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, float(scale), mask, int(size), sink,
-                                     q_lens, ctx_lens, out_dtype)
+                                     q_lens, ctx_lens, out_dtype, float(softcap), int(keep_first), talk)
     rep = H // G
     out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
     bs = rows.shape[1]
@@ -142,7 +145,9 @@ def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block
         p = pos[t0:t0 + n].long()
         sc = torch.einsum("thd,lhd->htl", q[t0:t0 + n], kk) * scale
         j = torch.arange(L, device=sc.device)[None, :]
-        vis = (j <= p[:, None]) & (j >= first_visible(p, mask, size)[:, None])
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
+        vis = (j <= p[:, None]) & ((j >= first_visible(p, mask, size)[:, None]) | (j < keep_first))
         sc = sc.masked_fill(~vis[None], float("-inf"))
         top = sc.max(-1, keepdim=True).values
         if sink is not None:
@@ -151,7 +156,10 @@ def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block
         den = e.sum(-1, keepdim=True)
         if sink is not None:
             den = den + torch.exp(sink.float()[:, None, None] - top)
-        out[t0:t0 + n] = torch.einsum("htl,lhd->thd", e / den, vv)
+        wts = e / den
+        if talk is not None:
+            wts = torch.einsum("hg,gtl->htl", talk.float(), wts)
+        out[t0:t0 + n] = torch.einsum("htl,lhd->thd", wts, vv)
         t0 += n
     return out.reshape(T, H * dv).to(out_dtype)
 

@@ -49,11 +49,23 @@ def rope_table(max_pos: int, dims: int, base: float, scaling: Optional[dict] = N
     With d(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(d(fast)), 0),
     hi = min(ceil(d(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 1e-3), 0, 1),
     pair i turns at f_i (1 - ramp_i) + f_i ramp_i / factor, and cos / sin carry
-    the magnitude 0.1 ln(factor) + 1."""
+    the magnitude 0.1 ln(factor) + 1.
+
+    ``scaling`` with the keys ``factor``, ``low``, ``high``, ``original`` (the
+    rule of Llama 3.1) acts on wavelengths l = 2 pi / f instead: f is kept where
+    l < original / high, divided by the factor where l > original / low, and in
+    between blended with s = (original / l - low) / (high - low) as
+    (1 - s) f / factor + s f."""
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = float(base) ** (-2.0 * i / dims)
     mag = 1.0
-    if scaling:
+    if scaling and "low" in scaling:
+        factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        orig = float(scaling["original"])
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - low) / (high - low) if high != low else torch.zeros_like(f)
+        f = torch.where(wl < orig / high, f, torch.where(wl > orig / low, f / factor, (1 - s) * f / factor + s * f))
+    elif scaling:
         factor = float(scaling["factor"])
 
         def d_of(t):
