@@ -81,7 +81,7 @@ def _cmd(src: str, obj: str):
             # some of them (profiles/gemv5_xm_forms_r6.txt)
             if os.path.basename(src) == "gemv_int4_xm.hip":
                 extra = ["-fno-slp-vectorize"]
-        if os.path.basename(src) in ("seqmix.hip", "ssm.hip", "maskattn.hip") or \
+        if os.path.basename(src) in ("seqmix.hip", "ssm.hip", "maskattn.hip", "gatedmix.hip") or \
                 os.path.basename(src).startswith("blockmix_"):
             # f32-exact kernels: no packed-f32 instruction forms
             extra = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -99,8 +99,9 @@ TARGETS = {
     # hybrid decoders: sequence-mixing kernels + their bindings + the serving scheduler
     # (+ the streaming skinny-GEMM kernel their decode-size projections share with the dense decoders)
     "seqmix": ["hip/seqmix.hip", "hip/blockmix_elem.hip", "hip/blockmix_attn.hip", "hip/blockmix_moe.hip",
-               "hip/ssm.hip", "hip/maskattn.hip", "hip/dense_gemv.hip", "torch/ops_seqmix.cpp",
-               "torch/ops_blockmix.cpp", "torch/ops_ssm.cpp", "torch/ops_maskattn.cpp", "torch/ops_dense.cpp",
+               "hip/ssm.hip", "hip/maskattn.hip", "hip/gatedmix.hip", "hip/dense_gemv.hip", "torch/ops_seqmix.cpp",
+               "torch/ops_blockmix.cpp", "torch/ops_ssm.cpp", "torch/ops_maskattn.cpp", "torch/ops_gatedmix.cpp",
+               "torch/ops_dense.cpp",
                "runtime/scheduler.cpp"],
 }
 

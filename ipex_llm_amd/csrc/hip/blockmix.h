@@ -67,15 +67,18 @@ void talk_softmax(bool bf16, float* sc, const int64_t* pos, int H, float scale, 
                   void* hi, void* lo, hipStream_t st);
 
 // ---- experts (blockmix_moe.hip)
-void moe_route(const float* z, int T, int E, int top, int32_t* idx, float* w, hipStream_t st);
+// mode 0: the largest sigmoid(z) win and are the weights; 1: the largest logits win, softmax over the winners (top <= 64)
+void moe_route(const float* z, int T, int E, int top, int32_t* idx, float* w, int mode, hipStream_t st);
 // off int32 [E + 1], sorted int32 [P]: pair ids (token * top + k) grouped by expert
 void moe_align(const int32_t* idx, int P, int E, int32_t* off, int32_t* sorted, hipStream_t st);
-// y [P, ff] (sorted order) = glu(W_gu[e] (w_p h_token))
+// y [P, ff] (sorted order) = glu(W_gu[e] (w_p h_token)), glu = g sigmoid(alpha g) (u + up_shift) with the clamps;
+// weigh_out: the input is h_token itself (the routing weight multiplies the result of moe_down instead)
 void moe_glu(bool bf16, const void* h, const int32_t* off, const int32_t* sorted, const float* wts, int top,
-             const void* w_gu, void* y, int P, int E, int ff, int W, float limit, float alpha, hipStream_t st);
-// out f32 [P, W] (by pair id) = W_down[e] y_p
+             const void* w_gu, void* y, int P, int E, int ff, int W, float limit, float alpha, float up_shift,
+             bool weigh_out, hipStream_t st);
+// out f32 [P, W] (by pair id) = W_down[e] y_p (times wts[pair] when wts is not null)
 void moe_down(bool bf16, const void* y, const int32_t* off, const int32_t* sorted, const void* w_down, float* out,
-              int P, int E, int ff, int W, hipStream_t st);
+              int P, int E, int ff, int W, const float* wts, hipStream_t st);
 
 }  // namespace bm
 }  // namespace illm

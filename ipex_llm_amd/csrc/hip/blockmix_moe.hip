@@ -1,7 +1,8 @@
 // Experts behind a sigmoid router (gfx950, wave64).
 //
 //   moe_route_k    sigmoid scores, the `top` largest per token (lowest index
-//                  first among equals) and those scores as weights
+//                  first among equals) and those scores as weights; or the
+//                  `top` largest logits and the softmax over them
 //   moe_align_k    pair ids (token * top + k) grouped by expert + offsets,
 //                  one workgroup, LDS counters: no host round trip, so a
 //                  step with experts can be captured in a hipGraph
@@ -34,18 +35,23 @@ template <> __device__ __forceinline__ float round_to<__bf16>(float v) { return 
 
 constexpr int kMaxPerLane = 8;      // experts <= 512
 
+// SOFTMAX false: scores sigmoid(z), the largest win and are the weights; true: the largest logits win, their weights
+// are the softmax over the winners only
+template <bool SOFTMAX>
 __global__ void __launch_bounds__(64) moe_route_k(const float* __restrict__ z, int E, int top, int32_t* __restrict__ idx,
                                                  float* __restrict__ w) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
+  const float none = SOFTMAX ? -INFINITY : -1.0f;                   // below every score; a taken one goes below that
   float s[kMaxPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxPerLane; i++) {
     const int e = lane + i * 64;
-    s[i] = e < E ? 1.0f / (1.0f + expf(-z[t * E + e])) : -1.0f;
+    s[i] = e < E ? (SOFTMAX ? fmaxf(z[t * E + e], -3.0e38f) : 1.0f / (1.0f + expf(-z[t * E + e]))) : none;
   }
+  float top0 = 0.f, den = 0.f, mine = 0.f;                          // SOFTMAX: lane k keeps winner k's weight (top <= 64)
   for (int k = 0; k < top; k++) {
-    float bv = -1.0f;
+    float bv = none;
     int be = 0x7fffffff;
 #pragma unroll
     for (int i = 0; i < kMaxPerLane; i++) {
@@ -64,14 +70,21 @@ __global__ void __launch_bounds__(64) moe_route_k(const float* __restrict__ z, i
         be = oe;
       }
     }
+    if (SOFTMAX) {                                                  // the first winner is the largest: exp(bv - top0) <= 1
+      if (k == 0) top0 = bv;
+      bv = expf(bv - top0);
+      den += bv;
+      if (lane == k) mine = bv;
+    }
     if (lane == 0) {
       idx[t * top + k] = be;
-      w[t * top + k] = bv;
+      if (!SOFTMAX) w[t * top + k] = bv;
     }
 #pragma unroll
     for (int i = 0; i < kMaxPerLane; i++)
-      if (lane + i * 64 == be) s[i] = -2.0f;
+      if (lane + i * 64 == be) s[i] = SOFTMAX ? -INFINITY : -2.0f;
   }
+  if (SOFTMAX && lane < top) w[t * top + lane] = mine / den;
 }
 
 __global__ void __launch_bounds__(1024) moe_align_k(const int32_t* __restrict__ idx, int P, int E, int32_t* __restrict__ off,
@@ -129,7 +142,7 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
                                                  const int32_t* __restrict__ sorted, const float* __restrict__ wts,
                                                  int top, const E* __restrict__ w, E* __restrict__ y,
                                                  float* __restrict__ outp, int nexp, int N, int K, float limit,
-                                                 float alpha) {
+                                                 float alpha, float up_shift, bool weigh_out) {
   __shared__ float xs[TM][TK + 1];
   __shared__ float ws[TN][TK + 1];
   __shared__ float ws2[GLU ? TN : 1][TK + 1];
@@ -145,7 +158,7 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
     if (sp < r1) {
       const int pid = sorted[sp];
       src_row[tid] = GLU ? pid / top : sp;
-      src_scale[tid] = GLU ? wts[pid] : 1.f;
+      src_scale[tid] = (GLU != weigh_out) ? wts[pid] : 1.f;         // GLU: on the input; DOWN (weigh_out): on the result
       dst_row[tid] = GLU ? sp : pid;
     } else {
       src_row[tid] = -1;
@@ -168,7 +181,7 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
       float v = 0.f;
       if (sr >= 0 && k0 + c < K) {
         v = ldf(x + (int64_t)sr * K + k0 + c);
-        if (GLU) v = round_to<E>(v * src_scale[r]);
+        if (GLU && !weigh_out) v = round_to<E>(v * src_scale[r]);
       }
       xs[r][c] = v;
     }
@@ -211,9 +224,9 @@ __global__ void __launch_bounds__(256) moe_gemm_k(const E* __restrict__ x, const
         // the products leave the matrix unit in the activation type, as a library product's would
         const float g = fminf(round_to<E>(acc[i][j]), limit);
         const float u = fminf(fmaxf(round_to<E>(acc2[i][j]), -limit), limit);
-        stf(y + (int64_t)dr * N + n, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+        stf(y + (int64_t)dr * N + n, g / (1.0f + expf(-alpha * g)) * (u + up_shift));
       } else {
-        outp[(int64_t)dr * N + n] = acc[i][j];
+        outp[(int64_t)dr * N + n] = weigh_out ? acc[i][j] * src_scale[ty * 2 + i] : acc[i][j];
       }
     }
   }
@@ -231,7 +244,7 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
                                                       const int32_t* __restrict__ sorted, const float* __restrict__ wts,
                                                       int top, const __bf16* __restrict__ w, __bf16* __restrict__ y,
                                                       float* __restrict__ outp, int nexp, int N, int K, float limit,
-                                                      float alpha) {
+                                                      float alpha, float up_shift, bool weigh_out) {
   constexpr int TKK = 64, AP = TKK + 8, MS = TMM / 16;
   __shared__ __attribute__((aligned(16))) __bf16 as[TMM * AP];
   __shared__ int src_row[TMM];
@@ -245,7 +258,7 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
     if (sp < r1) {
       const int pid = sorted[sp];
       src_row[tid] = GLU ? pid / top : sp;
-      src_scale[tid] = GLU ? wts[pid] : 1.f;
+      src_scale[tid] = (GLU != weigh_out) ? wts[pid] : 1.f;         // GLU: on the input; DOWN (weigh_out): on the result
       dst_row[tid] = GLU ? sp : pid;
     } else {
       src_row[tid] = -1;
@@ -295,7 +308,7 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
       const int c = tid + 256 * it;
       const int r = c >> 3, kc = (c & 7) * 8;
       bm_bf16x8 v = pa[it];
-      if (GLU) {
+      if (GLU && !weigh_out) {
         const float sc = src_scale[r];
 #pragma unroll
         for (int i = 0; i < 8; i++) v[i] = (__bf16)((float)v[i] * sc);
@@ -331,9 +344,9 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
       if (GLU) {
         const float gt = fminf((float)(__bf16)acc[m][i], limit);
         const float u = fminf(fmaxf((float)(__bf16)acc2[m][i], -limit), limit);
-        y[(int64_t)dr * N + col] = (__bf16)(gt / (1.0f + expf(-alpha * gt)) * (u + 1.0f));
+        y[(int64_t)dr * N + col] = (__bf16)(gt / (1.0f + expf(-alpha * gt)) * (u + up_shift));
       } else {
-        outp[(int64_t)dr * N + col] = acc[m][i];
+        outp[(int64_t)dr * N + col] = weigh_out ? acc[m][i] * src_scale[m * 16 + 4 * g + i] : acc[m][i];
       }
     }
   }
@@ -341,9 +354,10 @@ __global__ void __launch_bounds__(256) moe_gemm_mfma_k(const __bf16* __restrict_
 
 }  // namespace
 
-void moe_route(const float* z, int T, int E, int top, int32_t* idx, float* w, hipStream_t st) {
+void moe_route(const float* z, int T, int E, int top, int32_t* idx, float* w, int mode, hipStream_t st) {
   if (T <= 0) return;
-  moe_route_k<<<T, 64, 0, st>>>(z, E, top, idx, w);
+  if (mode == 1) moe_route_k<true><<<T, 64, 0, st>>>(z, E, top, idx, w);
+  else moe_route_k<false><<<T, 64, 0, st>>>(z, E, top, idx, w);
 }
 
 void moe_align(const int32_t* idx, int P, int E, int32_t* off, int32_t* sorted, hipStream_t st) {
@@ -351,41 +365,45 @@ void moe_align(const int32_t* idx, int P, int E, int32_t* off, int32_t* sorted, 
 }
 
 void moe_glu(bool bf16, const void* h, const int32_t* off, const int32_t* sorted, const float* wts, int top,
-             const void* w_gu, void* y, int P, int E, int ff, int W, float limit, float alpha, hipStream_t st) {
+             const void* w_gu, void* y, int P, int E, int ff, int W, float limit, float alpha, float up_shift,
+             bool weigh_out, hipStream_t st) {
   if (P <= 0) return;
   const dim3 grid((P + TM - 1) / TM + E, (ff + TN - 1) / TN);
   if (bf16 && W % 8 == 0) {
     if (P / E >= 64)
       moe_gemm_mfma_k<128, true><<<dim3((P + 127) / 128 + E, (ff + 63) / 64), 256, 0, st>>>(
-          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha);
+          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha, up_shift,
+          weigh_out);
     else
       moe_gemm_mfma_k<32, true><<<dim3((P + 31) / 32 + E, (ff + 63) / 64), 256, 0, st>>>(
-          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha);
+          (const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu, (__bf16*)y, nullptr, E, ff, W, limit, alpha, up_shift,
+          weigh_out);
   } else if (bf16)
     moe_gemm_k<__bf16, true><<<grid, 256, 0, st>>>((const __bf16*)h, off, sorted, wts, top, (const __bf16*)w_gu,
-                                                   (__bf16*)y, nullptr, E, ff, W, limit, alpha);
+                                                   (__bf16*)y, nullptr, E, ff, W, limit, alpha, up_shift, weigh_out);
   else
     moe_gemm_k<float, true><<<grid, 256, 0, st>>>((const float*)h, off, sorted, wts, top, (const float*)w_gu, (float*)y,
-                                                  nullptr, E, ff, W, limit, alpha);
+                                                  nullptr, E, ff, W, limit, alpha, up_shift, weigh_out);
 }
 
 void moe_down(bool bf16, const void* y, const int32_t* off, const int32_t* sorted, const void* w_down, float* out,
-              int P, int E, int ff, int W, hipStream_t st) {
+              int P, int E, int ff, int W, const float* wts, hipStream_t st) {
+  const bool wo = wts != nullptr;                                   // the routing weight multiplies the result row
   if (P <= 0) return;
   const dim3 grid((P + TM - 1) / TM + E, (W + TN - 1) / TN);
   if (bf16 && ff % 8 == 0) {
     if (P / E >= 64)
       moe_gemm_mfma_k<128, false><<<dim3((P + 127) / 128 + E, (W + 63) / 64), 256, 0, st>>>(
-          (const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f);
+          (const __bf16*)y, off, sorted, wts, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f, 0.f, wo);
     else
       moe_gemm_mfma_k<32, false><<<dim3((P + 31) / 32 + E, (W + 63) / 64), 256, 0, st>>>(
-          (const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f);
+          (const __bf16*)y, off, sorted, wts, 1, (const __bf16*)w_down, nullptr, out, E, W, ff, 0.f, 0.f, 0.f, wo);
   } else if (bf16)
-    moe_gemm_k<__bf16, false><<<grid, 256, 0, st>>>((const __bf16*)y, off, sorted, nullptr, 1, (const __bf16*)w_down,
-                                                    nullptr, out, E, W, ff, 0.f, 0.f);
+    moe_gemm_k<__bf16, false><<<grid, 256, 0, st>>>((const __bf16*)y, off, sorted, wts, 1, (const __bf16*)w_down,
+                                                    nullptr, out, E, W, ff, 0.f, 0.f, 0.f, wo);
   else
-    moe_gemm_k<float, false><<<grid, 256, 0, st>>>((const float*)y, off, sorted, nullptr, 1, (const float*)w_down,
-                                                   nullptr, out, E, W, ff, 0.f, 0.f);
+    moe_gemm_k<float, false><<<grid, 256, 0, st>>>((const float*)y, off, sorted, wts, 1, (const float*)w_down,
+                                                   nullptr, out, E, W, ff, 0.f, 0.f, 0.f, wo);
 }
 
 }  // namespace bm

@@ -67,16 +67,17 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // ------------------------------------------------------------------ norm + rotary + append
 // hs: LDS [H + G] sums of squares per head
-template <typename E>
-__device__ __forceinline__ float normed(const E* x, int i, int head, int d, const E* nw, bool whole, float rs) {
+template <typename EI, typename E>
+__device__ __forceinline__ float normed(const EI* x, int i, int head, int d, const E* nw, bool whole, float rs) {
   float v = ldf(x + i);
   if (nw) v = v * rs * ldf(nw + (whole ? head * d + i : i));
   return v;
 }
 
-template <typename E>
-__global__ void __launch_bounds__(1024) qkv_store_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
-                                                  int64_t k_ld, const E* __restrict__ v, int64_t v_ld,
+// EI: element type of the projected q / k / v (f32 when a convolution came first), E: of the norm weights and the rows
+template <typename EI, typename E>
+__global__ void __launch_bounds__(1024) qkv_store_k(const EI* __restrict__ q, int64_t q_ld, const EI* __restrict__ k,
+                                                  int64_t k_ld, const EI* __restrict__ v, int64_t v_ld,
                                                   const E* __restrict__ qn, const E* __restrict__ kn, bool whole,
                                                   float eps, const float* __restrict__ table, int dims, int layout,
                                                   const int64_t* __restrict__ pos, const int64_t* __restrict__ slots,
@@ -86,10 +87,10 @@ __global__ void __launch_bounds__(1024) qkv_store_k(const E* __restrict__ q, int
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
   const int NH = H + (k ? G : 0);
-  const E* qr = q + t * q_ld;
-  const E* kr = k ? k + t * k_ld : nullptr;
+  const EI* qr = q + t * q_ld;
+  const EI* kr = k ? k + t * k_ld : nullptr;
   for (int hh = wv; hh < NH; hh += NW) {
-    const E* x = hh < H ? qr + hh * d : kr + (hh - H) * d;
+    const EI* x = hh < H ? qr + hh * d : kr + (hh - H) * d;
     float s = 0.f;
     for (int i = lane; i < d; i += 64) {
       const float a = ldf(x + i);
@@ -115,7 +116,7 @@ __global__ void __launch_bounds__(1024) qkv_store_k(const E* __restrict__ q, int
     const int hh = e / d, i = e - hh * d;
     const bool isq = hh < H;
     const int head = isq ? hh : hh - H;
-    const E* x = isq ? qr + head * d : kr + head * d;
+    const EI* x = isq ? qr + head * d : kr + head * d;
     const E* nw = isq ? qn : kn;
     float rs = 1.f;
     if (nw) rs = whole ? 1.0f / sqrtf(hs[isq ? NH : NH + 1] / (float)((isq ? H : G) * d) + eps)
@@ -141,7 +142,7 @@ __global__ void __launch_bounds__(1024) qkv_store_k(const E* __restrict__ q, int
     else stf(row + head * d + i, val);
   }
   if (k)
-    for (int e = threadIdx.x; e < G * dv; e += blockDim.x) row[(int64_t)G * d + e] = v[t * v_ld + e];
+    for (int e = threadIdx.x; e < G * dv; e += blockDim.x) stf(row + (int64_t)G * d + e, ldf(v + t * v_ld + e));
 }
 
 // ------------------------------------------------------------------ attention
@@ -164,13 +165,17 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
                                                     const int32_t* __restrict__ seq_of, const int64_t* __restrict__ pos,
                                                     float scale, int mask, int size, const float* __restrict__ sink,
                                                     E* __restrict__ out, float* __restrict__ part, int H, int G, int d,
-                                                    int dv, int DQ, int DP) {
+                                                    int dv, int DQ, int DP, float softcap, int keep, int cross) {
   extern __shared__ __align__(16) unsigned char smem[];
   typedef typename Chunk4<E>::type C4;
   const int rep = H / G;
   const int nhb = (rep + HB - 1) / HB;                              // head blocks per key head
   const int nsplit = gridDim.z, zs = blockIdx.z;
-  const int t = blockIdx.x, g = blockIdx.y / nhb, h0 = g * rep + (blockIdx.y % nhb) * HB;
+  // cross: the heads' weights are applied to the values of EVERY value head (grid y also walks the value heads); the
+  // unnormalised partial results leave through ``part`` and the mixing of the heads follows in the combine kernel
+  const int by = cross ? blockIdx.y / G : blockIdx.y;
+  const int t = blockIdx.x, g = by / nhb, h0 = g * rep + (by % nhb) * HB;
+  const int vg = cross ? blockIdx.y % G : g;
   const int nh = min(HB, g * rep + rep - h0);
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
   float* qs = (float*)smem;
@@ -190,6 +195,9 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
   const int64_t lo = first_key(p, mask, size);
   const int32_t* tab = bt + (int64_t)seq_of[t] * bt_w;
   const int tile0 = (int)(lo / KT), ntiles = (int)(p / KT) + 1;
+  // a window that keeps the sequence's first tokens: their tiles (those before the window's first) are walked first
+  const int nkeep = keep > 0 ? min(tile0, (keep + KT - 1) / KT) : 0;
+  const int nwalk = nkeep + ntiles - tile0;
   const int64_t RW = (int64_t)G * (d + dv);                         // cache row width
   const int D = d + dv;
   float m[HB], l[HB], o[HB][RC];
@@ -202,7 +210,8 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
   }
   const int kj = lane & (KT - 1), grp = lane / KT;                  // 4 lanes share a key
   const int d4 = (d + 3) >> 2;                                      // 4-element steps of a key (LDS pad is zero)
-  for (int ti = tile0 + zs * NW + wv; ti < ntiles; ti += NW * nsplit) {
+  for (int it = zs * NW + wv; it < nwalk; it += NW * nsplit) {
+    const int ti = it < nkeep ? it : tile0 + (it - nkeep);
     const int64_t k0 = (int64_t)ti * KT;
     const int nvalid = (int)min((int64_t)KT, p - k0 + 1);
     const int64_t row0 = (int64_t)tab[k0 / bs] * bs + (k0 % bs);
@@ -218,7 +227,7 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
           if (i < n4) {
             const int j = i / cpr, c = i - j * cpr;
             const E* src = rows + (row0 + j) * RW +
-                           (c < cd ? (int64_t)g * d + 4 * c : (int64_t)G * d + (int64_t)g * dv + 4 * (c - cd));
+                           (c < cd ? (int64_t)g * d + 4 * c : (int64_t)G * d + (int64_t)vg * dv + 4 * (c - cd));
             v[u] = *(const C4*)src;
             dst[u] = j * DP + (c < cd ? 4 * c : DQ + 4 * (c - cd));
           }
@@ -230,7 +239,7 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
     } else {
       for (int i = lane; i < nvalid * D; i += 64) {
         const int j = i / D, c = i - j * D;
-        const E* src = rows + (row0 + j) * RW + (c < d ? (int64_t)g * d + c : (int64_t)G * d + (int64_t)g * dv + (c - d));
+        const E* src = rows + (row0 + j) * RW + (c < d ? (int64_t)g * d + c : (int64_t)G * d + (int64_t)vg * dv + (c - d));
         kt[j * DP + (c < d ? c : DQ + (c - d))] = *src;
       }
     }
@@ -238,7 +247,7 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
     float s[HB];
 #pragma unroll
     for (int h = 0; h < HB; h++) s[h] = 0.f;
-    const bool valid = kj < nvalid && k0 + kj >= lo;
+    const bool valid = kj < nvalid && (k0 + kj >= lo || k0 + kj < keep);
     if (valid) {
       const E* kr = kt + kj * DP;
       for (int c4 = grp * d4 / 4; c4 < (grp + 1) * d4 / 4; c4++) {
@@ -258,7 +267,9 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
     }
 #pragma unroll
     for (int h = 0; h < HB; h++) {
-      const float sv = valid ? s[h] * scale : -INFINITY;
+      float sv = s[h] * scale;
+      if (softcap > 0.f) sv = softcap * tanhf(sv / softcap);
+      if (!valid) sv = -INFINITY;
       const float mn = fmaxf(m[h], wave_max(sv));
       const float alpha = m[h] == -INFINITY ? 0.f : expf(m[h] - mn);
       const float pv = valid ? expf(sv - mn) : 0.f;
@@ -319,7 +330,10 @@ __global__ void __launch_bounds__(256) masked_attn_k(const float* __restrict__ q
       L += gp[dv + 1] * f;
       if (c < dv) O += gp[c] * f;
     }
-    if (nsplit > 1) {
+    if (cross) {
+      float* pp = part + ((((int64_t)t * H + h0 + h) * G + vg) * nsplit + zs) * (dv + 2);
+      pp[c] = c < dv ? O : (c == dv ? M : L);
+    } else if (nsplit > 1) {
       float* pp = part + (((int64_t)t * H + h0 + h) * nsplit + zs) * (dv + 2);
       pp[c] = c < dv ? O : (c == dv ? M : L);
     } else if (c < dv) {
@@ -362,10 +376,86 @@ __global__ void __launch_bounds__(64) masked_attn_combine_k(const float* __restr
   }
 }
 
+// merge of the key splits and mixing of the heads' weights after the softmax:
+//   out[t, h] = sum_g talk[h, g] (sum_j w_g(j) value_j[c])   with c = h's value head,
+// part [T, H, G, nsplit, dv + 2] holds, for query head g and value head c, the unnormalised sums of every key split.
+// One wave per (token, output head); dv <= 512
+template <typename E>
+__global__ void __launch_bounds__(64) masked_attn_talk_combine_k(const float* __restrict__ part,
+                                                                const float* __restrict__ sink,
+                                                                const float* __restrict__ talk, E* __restrict__ out,
+                                                                int H, int G, int dv, int nsplit) {
+  __shared__ float wz[64];
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, c = h / (H / G), lane = threadIdx.x;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = 0.f;
+  for (int g = 0; g < H; g++) {
+    const float* pp = part + ((t * H + g) * G + c) * (int64_t)nsplit * (dv + 2);
+    const float mz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv] : -INFINITY;
+    const float lz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
+    const float sk = sink ? sink[g] : -INFINITY;
+    const float M = fmaxf(wave_max(mz), sk);
+    const float f = mz == -INFINITY ? 0.f : expf(mz - M);
+    __syncthreads();
+    wz[lane] = f;
+    __syncthreads();
+    float L = sink ? expf(sk - M) : 0.f;
+    for (int z = 0; z < nsplit; z++) L += __shfl(lz, z, 64) * wz[z];   // index order, whatever the lanes do
+    const float coef = talk[h * H + g] / L;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int col = lane + 64 * i;
+      if (col < dv) {
+        float O = 0.f;
+        for (int z = 0; z < nsplit; z++) O = fmaf(pp[(size_t)z * (dv + 2) + col], wz[z], O);
+        acc[i] = fmaf(coef, O, acc[i]);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int col = lane + 64 * i;
+    if (col < dv) stf(out + (t * H + h) * dv + col, acc[i]);
+  }
+}
+
+// mixing of the heads' weights between the chunk products: w f32 [pieces, G, Lq, rep, L] (normalised softmax
+// weights) -> mixed weights of the same layout, w'[.., h, ..] = sum_g talk[h, g] w[.., g, ..] with h = key head * rep +
+// r; bf16: as pairs hi + lo in hl [R, 2 L] (a row's hi halves, then its lo halves); f32: out32 [R, L].
+// A thread per key column, the piece-and-query's H weights of that column staged in LDS
+template <typename E>
+__global__ void __launch_bounds__(64) talk_mix_k(const float* __restrict__ w, const float* __restrict__ talk, int Lq, int L,
+                                                int G, int rep, E* __restrict__ hl, float* __restrict__ out32) {
+  extern __shared__ float col[];                                    // [H][64]
+  const int H = G * rep;
+  const int piece = blockIdx.x / Lq, qi = blockIdx.x % Lq;
+  const int j = blockIdx.y * 64 + threadIdx.x;
+  if (j >= L) return;
+  const int64_t prow = (int64_t)piece * G * Lq * rep;
+  for (int g = 0; g < H; g++) {
+    const int64_t row = prow + ((int64_t)(g / rep) * Lq + qi) * rep + g % rep;
+    col[g * 64 + threadIdx.x] = w[row * L + j];
+  }
+  for (int h = 0; h < H; h++) {
+    float a = 0.f;
+    for (int g = 0; g < H; g++) a = fmaf(talk[h * H + g], col[g * 64 + threadIdx.x], a);
+    const int64_t row = prow + ((int64_t)(h / rep) * Lq + qi) * rep + h % rep;
+    if (hl) {
+      const E hv = (E)a;
+      hl[row * 2 * L + j] = hv;
+      hl[row * 2 * L + L + j] = (E)(a - (float)hv);
+    } else {
+      out32[row * L + j] = a;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ softmax between the chunk products
 template <typename E>
 __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, int Lq, int L, int G, int rep, float scale,
-                                                      const float* __restrict__ sink, E* __restrict__ hi) {
+                                                      const float* __restrict__ sink, E* __restrict__ hi, float softcap) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
   const int tok = (int)((row / rep) % Lq);                          // the piece's queries are its last Lq positions
@@ -374,7 +464,12 @@ __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, i
   float* s = sc + row * L;
   const float sk = sink ? sink[h] : -INFINITY;
   float mx = sk;
-  for (int j = threadIdx.x; j < nk; j += blockDim.x) mx = fmaxf(mx, s[j] * scale);
+  for (int j = threadIdx.x; j < nk; j += blockDim.x) {
+    float v = s[j] * scale;
+    if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+    s[j] = v;
+    mx = fmaxf(mx, v);
+  }
   mx = wave_max(mx);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
@@ -382,7 +477,7 @@ __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, i
   for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
   float sum = 0.f;
   for (int j = threadIdx.x; j < nk; j += blockDim.x) {
-    const float e = expf(s[j] * scale - mx);
+    const float e = expf(s[j] - mx);
     s[j] = e;
     sum += e;
   }
@@ -418,10 +513,10 @@ int tile_row(int d, int dv) {
 
 }  // namespace
 
-void qkv_norm_rope_store(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v,
-                         int64_t v_ld, const void* qn, const void* kn, bool whole, float eps, const float* table,
-                         int max_pos, int dims, int layout, const int64_t* pos, const int64_t* slots, void* rows,
-                         int64_t num_rows, float* qo, int T, int H, int G, int d, int dv, hipStream_t st) {
+void qkv_norm_rope_store(bool in_bf16, bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_ld,
+                         const void* v, int64_t v_ld, const void* qn, const void* kn, bool whole, float eps,
+                         const float* table, int max_pos, int dims, int layout, const int64_t* pos, const int64_t* slots,
+                         void* rows, int64_t num_rows, float* qo, int T, int H, int G, int d, int dv, hipStream_t st) {
   (void)max_pos;
   (void)num_rows;
   if (T <= 0) return;
@@ -429,14 +524,14 @@ void qkv_norm_rope_store(bool bf16, const void* q, int64_t q_ld, const void* k, 
   // few tokens (decode): a thread per value or two, so that no thread walks a chain of dependent loads
   const int64_t vals = (int64_t)(H + G) * d;
   const int nt = T > 64 ? 256 : (vals >= 1024 ? 1024 : (int)((vals + 63) / 64 * 64));
-  if (bf16)
-    qkv_store_k<__bf16><<<T, nt, lds, st>>>((const __bf16*)q, q_ld, (const __bf16*)k, k_ld, (const __bf16*)v, v_ld,
-                                             (const __bf16*)qn, (const __bf16*)kn, whole, eps, table, dims, layout, pos,
-                                             slots, (__bf16*)rows, qo, H, G, d, dv);
-  else
-    qkv_store_k<float><<<T, nt, lds, st>>>((const float*)q, q_ld, (const float*)k, k_ld, (const float*)v, v_ld,
-                                            (const float*)qn, (const float*)kn, whole, eps, table, dims, layout, pos,
-                                            slots, (float*)rows, qo, H, G, d, dv);
+#define MA_STORE(EI, E)                                                                                                 \
+  qkv_store_k<EI, E><<<T, nt, lds, st>>>((const EI*)q, q_ld, (const EI*)k, k_ld, (const EI*)v, v_ld, (const E*)qn,      \
+                                         (const E*)kn, whole, eps, table, dims, layout, pos, slots, (E*)rows, qo, H, G, \
+                                         d, dv)
+  if (bf16 && in_bf16) MA_STORE(__bf16, __bf16);
+  else if (bf16) MA_STORE(float, __bf16);
+  else MA_STORE(float, float);
+#undef MA_STORE
 }
 
 int masked_attention_plan(bool bf16, int rep, int d, int dv, int* nw, int* hbo) {
@@ -458,10 +553,10 @@ int masked_attention_plan(bool bf16, int rep, int d, int dv, int* nw, int* hbo) 
   return -1;
 }
 
-int masked_attention_splits(bool bf16, int T, int H, int G, int d, int dv, int max_keys) {
+int masked_attention_splits(bool bf16, int T, int H, int G, int d, int dv, int max_keys, bool cross) {
   int NW = 0, hb = 0;
   if (masked_attention_plan(bf16, H / G, d, dv, &NW, &hb) < 0) return 1;
-  const int64_t blocks = (int64_t)T * G * ((H / G + hb - 1) / hb);
+  const int64_t blocks = (int64_t)T * G * ((H / G + hb - 1) / hb) * (cross ? G : 1);
   const int tiles = (max_keys + KT - 1) / KT + 1;
   int ns = (int)((1024 + blocks - 1) / blocks);                    // ~4 workgroups per CU
   ns = ns > (tiles + NW - 1) / NW ? (tiles + NW - 1) / NW : ns;
@@ -470,18 +565,22 @@ int masked_attention_splits(bool bf16, int T, int H, int G, int d, int dv, int m
 
 void masked_attention(bool bf16, const float* q, const void* rows, int bs, const int32_t* block_tables, int bt_width,
                       const int32_t* seq_of, const int64_t* pos, float scale, int mask, int size, const float* sink,
-                      void* out, float* part, int nsplit, int T, int H, int G, int d, int dv, hipStream_t st) {
+                      void* out, float* part, int nsplit, int T, int H, int G, int d, int dv, float softcap, int keep,
+                      const float* talk, hipStream_t st) {
   if (T <= 0) return;
+  const int cross = talk ? 1 : 0;
+  if (mask != kWindow) keep = 0;
   int NW = 0, hb = 0;
   const int rep = H / G;
   const int lds = masked_attention_plan(bf16, rep, d, dv, &NW, &hb);
   if (lds < 0) return;                       // refused by the caller beforehand
   const int DQ = pad4(d), DP = tile_row(d, dv);
   const int rc = (dv + 63) / 64;
-  dim3 grid(T, G * ((rep + hb - 1) / hb), nsplit), block(64 * NW);
+  dim3 grid(T, G * ((rep + hb - 1) / hb) * (cross ? G : 1), nsplit), block(64 * NW);
 #define MA_LAUNCH(E, RC, HBV)                                                                                          \
   masked_attn_k<E, RC, HBV><<<grid, block, lds, st>>>(q, (const E*)rows, bs, block_tables, bt_width, seq_of, pos, scale, \
-                                                      mask, size, sink, (E*)out, part, H, G, d, dv, DQ, DP)
+                                                      mask, size, sink, (E*)out, part, H, G, d, dv, DQ, DP, softcap,   \
+                                                      keep, cross)
 #define MA_RC(E, HBV)                                 \
   if (rc <= 1) MA_LAUNCH(E, 1, HBV);                  \
   else if (rc <= 2) MA_LAUNCH(E, 2, HBV);             \
@@ -496,17 +595,29 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
 #undef MA_HB
 #undef MA_RC
 #undef MA_LAUNCH
-  if (nsplit > 1) {
+  if (cross) {
+    if (bf16) masked_attn_talk_combine_k<__bf16><<<dim3(T, H), 64, 0, st>>>(part, sink, talk, (__bf16*)out, H, G, dv, nsplit);
+    else masked_attn_talk_combine_k<float><<<dim3(T, H), 64, 0, st>>>(part, sink, talk, (float*)out, H, G, dv, nsplit);
+  } else if (nsplit > 1) {
     if (bf16) masked_attn_combine_k<__bf16><<<dim3(T, H), 64, 0, st>>>(part, sink, (__bf16*)out, H, dv, nsplit);
     else masked_attn_combine_k<float><<<dim3(T, H), 64, 0, st>>>(part, sink, (float*)out, H, dv, nsplit);
   }
 }
 
 void chunk_softmax(bool bf16, float* sc, int64_t R, int Lq, int L, int G, int rep, float scale, const float* sink,
-                   void* hl, hipStream_t st) {
+                   void* hl, float softcap, hipStream_t st) {
   if (R <= 0 || L <= 0) return;
-  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (__bf16*)hl);
-  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (float*)nullptr);
+  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (__bf16*)hl, softcap);
+  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (float*)nullptr, softcap);
+}
+
+void talk_mix(bool bf16, const float* w, const float* talk, int64_t pieces, int Lq, int L, int G, int rep, void* hl,
+              float* out32, hipStream_t st) {
+  if (pieces <= 0 || L <= 0) return;
+  const dim3 grid((unsigned)(pieces * Lq), (L + 63) / 64);
+  const size_t lds = (size_t)G * rep * 64 * sizeof(float);
+  if (bf16) talk_mix_k<__bf16><<<grid, 64, lds, st>>>(w, talk, Lq, L, G, rep, (__bf16*)hl, nullptr);
+  else talk_mix_k<float><<<grid, 64, lds, st>>>(w, talk, Lq, L, G, rep, (float*)nullptr, out32);
 }
 
 void sigmoid_gate(bool bf16, void* o, const void* g, int64_t g_ld, int64_t T, int C, hipStream_t st) {

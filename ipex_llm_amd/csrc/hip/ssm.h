@@ -10,12 +10,13 @@
 namespace illm {
 namespace ssm {
 
-// out f32 [T, C] = silu(b + sum_j w[:, j] u_(t - taps + 1 + j)); u rows of u_ld elements; w f32 [C, taps], b f32 [C];
+// out f32 [T, C] = silu(b + sum_j w[:, j] u_(t - taps + 1 + j)) (b null: no bias; act false: no SiLU); u rows of u_ld
+// elements; w f32 [C, taps], b f32 [C];
 // state f32 [slots, taps - 1, C], advanced afterwards (by the same launch when ``single``: every sequence brings
 // exactly one token)
 void conv_silu(bool bf16, const void* u, int64_t u_ld, const float* w, const float* b, int taps, float* state,
                const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* out, int T,
-               int B, int C, bool single, hipStream_t st);
+               int B, int C, bool single, bool act, hipStream_t st);
 
 // largest state size N the scan holds
 constexpr int kScanMaxState = 1024;

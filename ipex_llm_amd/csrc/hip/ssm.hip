@@ -77,7 +77,8 @@ template <> __device__ __forceinline__ void stv<4>(float* p, const float* v) {
   *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
 }
 
-template <typename E, int V>
+// bias may be null; ACT: SiLU on the result
+template <typename E, int V, bool ACT>
 __global__ void __launch_bounds__(256) conv_silu_k(const E* __restrict__ u, int64_t u_ld, const float* __restrict__ w,
                                                   const float* __restrict__ bias, int taps, float* __restrict__ state,
                                                   const int32_t* __restrict__ cu, const int32_t* __restrict__ seq_of,
@@ -91,7 +92,9 @@ __global__ void __launch_bounds__(256) conv_silu_k(const E* __restrict__ u, int6
   const int64_t p = pos[t];
   float* st = state + (int64_t)slots[b] * (taps - 1) * C + c;       // [taps - 1][C], oldest first
   float acc[V];
-  LdV<float, V>::ld(bias + c, acc);
+#pragma unroll
+  for (int q = 0; q < V; q++) acc[q] = 0.f;
+  if (bias) LdV<float, V>::ld(bias + c, acc);
   for (int j = 0; j < taps; j++) {
     const int back = taps - 1 - j;                                  // the input of position p - back
     float v[V];
@@ -102,8 +105,10 @@ __global__ void __launch_bounds__(256) conv_silu_k(const E* __restrict__ u, int6
 #pragma unroll
     for (int q = 0; q < V; q++) acc[q] = fmaf(w[(int64_t)(c + q) * taps + j], v[q], acc[q]);
   }
+  if (ACT) {
 #pragma unroll
-  for (int q = 0; q < V; q++) acc[q] = silu(acc[q]);
+    for (int q = 0; q < V; q++) acc[q] = silu(acc[q]);
+  }
   stv<V>(out + (int64_t)t * C + c, acc);
   if (single && taps > 1) {
     // the only token of its sequence (i == 0): the slot moves up by one position; row j held position
@@ -303,21 +308,26 @@ __global__ void __launch_bounds__(256) gated_group_norm_k(const float* __restric
 
 void conv_silu(bool bf16, const void* u, int64_t u_ld, const float* w, const float* b, int taps, float* state,
                const int32_t* cu, const int32_t* seq_of, const int32_t* slots, const int64_t* pos, float* out, int T,
-               int B, int C, bool single, hipStream_t st) {
+               int B, int C, bool single, bool act, hipStream_t st) {
   if (T <= 0 || C <= 0) return;
   const size_t eb = bf16 ? 2 : 4;
   const bool v4 = (C & 3) == 0 && (u_ld & 3) == 0 && ((uintptr_t)u % (4 * eb)) == 0;
   const int cw = v4 ? C / 4 : C;
   dim3 grid(T, (cw + 255) / 256), gs(B, (C + 255) / 256);
 #define SSM_CONV(E, V)                                                                                               \
-  conv_silu_k<E, V><<<grid, 256, 0, st>>>((const E*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, C, single)
+  if (act)                                                                                                           \
+    conv_silu_k<E, V, true><<<grid, 256, 0, st>>>((const E*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, \
+                                                  C, single);                                                        \
+  else                                                                                                               \
+    conv_silu_k<E, V, false><<<grid, 256, 0, st>>>((const E*)u, u_ld, w, b, taps, state, cu, seq_of, slots, pos, out, \
+                                                   C, single)
   if (bf16) {
-    if (v4) SSM_CONV(__bf16, 4);
-    else SSM_CONV(__bf16, 1);
+    if (v4) { SSM_CONV(__bf16, 4); }
+    else { SSM_CONV(__bf16, 1); }
     if (!single && taps > 1) conv_state_k<__bf16><<<gs, 256, 0, st>>>((const __bf16*)u, u_ld, taps, state, cu, slots, pos, C);
   } else {
-    if (v4) SSM_CONV(float, 4);
-    else SSM_CONV(float, 1);
+    if (v4) { SSM_CONV(float, 4); }
+    else { SSM_CONV(float, 1); }
     if (!single && taps > 1) conv_state_k<float><<<gs, 256, 0, st>>>((const float*)u, u_ld, taps, state, cu, slots, pos, C);
   }
 #undef SSM_CONV

@@ -357,20 +357,21 @@ std::tuple<Tensor, Tensor> bm_talk_softmax(Tensor& sc, const Tensor& pos, int64_
   return {hi, lo};
 }
 
-std::tuple<Tensor, Tensor> bm_moe_route(const Tensor& z, int64_t top) {
+std::tuple<Tensor, Tensor> bm_moe_route(const Tensor& z, int64_t top, int64_t mode) {
   c10::DeviceGuard g(z.device());
   check_f32_rows(z, "bm_moe_route: router logits f32 [T, E]");
   const int64_t T = z.size(0), E = z.size(1);
   TORCH_CHECK(E >= 1 && E <= 512 && top >= 1 && top <= E, "bm_moe_route: 1 <= top <= experts <= 512");
+  TORCH_CHECK(mode == 0 || (mode == 1 && top <= 64), "bm_moe_route: mode 0 (sigmoid) or 1 (softmax over the chosen, top <= 64)");
   Tensor idx = at::empty({T, top}, z.options().dtype(at::kInt));
   Tensor w = at::empty({T, top}, z.options());
   illm::bm::moe_route(z.data_ptr<float>(), (int)T, (int)E, (int)top, idx.data_ptr<int32_t>(), w.data_ptr<float>(),
-                      stream());
+                      (int)mode, stream());
   return {idx, w};
 }
 
 Tensor bm_moe_experts(const Tensor& h, const Tensor& idx, const Tensor& wts, const Tensor& w_gu, const Tensor& w_down,
-                      double limit, double alpha) {
+                      double limit, double alpha, double up_shift, bool weigh_out) {
   c10::DeviceGuard g(h.device());
   TORCH_CHECK(h.is_cuda() && h.dim() == 2 && is_act(h) && h.is_contiguous(), "bm_moe_experts: h [T, W] contiguous");
   const int64_t T = h.size(0), W = h.size(1);
@@ -397,9 +398,10 @@ Tensor bm_moe_experts(const Tensor& h, const Tensor& idx, const Tensor& wts, con
   illm::bm::moe_align(idx.data_ptr<int32_t>(), (int)P, (int)E, off.data_ptr<int32_t>(), sorted.data_ptr<int32_t>(), st);
   illm::bm::moe_glu(bf(h), h.data_ptr(), off.data_ptr<int32_t>(), sorted.data_ptr<int32_t>(), wts.data_ptr<float>(),
                     (int)top, w_gu.data_ptr(), y.data_ptr(), (int)P, (int)E, (int)ff, (int)W, (float)limit,
-                    (float)alpha, st);
+                    (float)alpha, (float)up_shift, weigh_out, st);
   illm::bm::moe_down(bf(h), y.data_ptr(), off.data_ptr<int32_t>(), sorted.data_ptr<int32_t>(), w_down.data_ptr(),
-                     out.data_ptr<float>(), (int)P, (int)E, (int)ff, (int)W, st);
+                     out.data_ptr<float>(), (int)P, (int)E, (int)ff, (int)W, weigh_out ? wts.data_ptr<float>() : nullptr,
+                     st);
   if (top == 1) return out;
   return out.view({T, top, W}).sum(1);
 }
@@ -429,9 +431,9 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
         "Tensor? talk, Tensor? gate, int G, Tensor(a!) out) -> ()");
   m.def("bm_talk_softmax(Tensor(a!) scores, Tensor pos, int H, float scale, Tensor? talk, bool act_f32) -> "
         "(Tensor, Tensor)");
-  m.def("bm_moe_route(Tensor z, int top) -> (Tensor, Tensor)");
-  m.def("bm_moe_experts(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_down, float limit, float alpha) -> "
-        "Tensor");
+  m.def("bm_moe_route(Tensor z, int top, int mode) -> (Tensor, Tensor)");
+  m.def("bm_moe_experts(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_down, float limit, float alpha, "
+        "float up_shift, bool weigh_out) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(ipex_llm_amd, CompositeExplicitAutograd, m) {

@@ -23,8 +23,8 @@ void check_f32_vec(const Tensor& t, int64_t n, const char* what) {
   TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous() && t.numel() == n, what);
 }
 
-Tensor ssm_conv_silu(const Tensor& u, const Tensor& w, const Tensor& b, Tensor& state, const Tensor& cu,
-                     const Tensor& seq_of, const Tensor& slots, const Tensor& pos, bool single) {
+Tensor ssm_conv_silu(const Tensor& u, const Tensor& w, const c10::optional<Tensor>& b, Tensor& state, const Tensor& cu,
+                     const Tensor& seq_of, const Tensor& slots, const Tensor& pos, bool single, bool act) {
   c10::DeviceGuard g(u.device());
   TORCH_CHECK(u.is_cuda() && u.dim() == 2 && is_act(u) && (u.size(1) <= 1 || u.stride(1) == 1) && u.stride(0) >= u.size(1),
               "ssm_conv_silu: u [T, C] (unit inner stride)");
@@ -33,7 +33,8 @@ Tensor ssm_conv_silu(const Tensor& u, const Tensor& w, const Tensor& b, Tensor& 
                   w.size(1) >= 1 && w.size(1) <= 16,
               "ssm_conv_silu: w f32 [C, taps], 1 <= taps <= 16");
   const int64_t taps = w.size(1);
-  check_f32_vec(b, C, "ssm_conv_silu: bias f32 [C]");
+  const bool has_b = b.has_value() && b->defined();
+  if (has_b) check_f32_vec(*b, C, "ssm_conv_silu: bias f32 [C]");
   TORCH_CHECK(state.is_cuda() && state.scalar_type() == at::kFloat && state.is_contiguous() && state.dim() == 3 &&
                   state.size(1) == taps - 1 && state.size(2) == C,
               "ssm_conv_silu: state f32 [slots, taps - 1, C]");
@@ -46,10 +47,10 @@ Tensor ssm_conv_silu(const Tensor& u, const Tensor& w, const Tensor& b, Tensor& 
   check_idx(slots, at::kInt, B, "ssm_conv_silu: state slots int32 [B]");
   check_idx(pos, at::kLong, T, "ssm_conv_silu: pos int64 [T]");
   Tensor out = at::empty({T, C}, u.options().dtype(at::kFloat));
-  illm::ssm::conv_silu(bf(u), u.data_ptr(), u.stride(0), w.data_ptr<float>(), b.data_ptr<float>(), (int)taps,
+  illm::ssm::conv_silu(bf(u), u.data_ptr(), u.stride(0), w.data_ptr<float>(), has_b ? b->data_ptr<float>() : nullptr, (int)taps,
                        state.data_ptr<float>(), cu.data_ptr<int32_t>(), seq_of.data_ptr<int32_t>(),
                        slots.data_ptr<int32_t>(), pos.data_ptr<int64_t>(), out.data_ptr<float>(), (int)T, (int)B, (int)C,
-                       single, stream());
+                       single, act, stream());
   return out;
 }
 
@@ -114,8 +115,8 @@ Tensor ssm_gated_group_norm(const Tensor& y, const Tensor& z, const Tensor& w, i
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
-  m.def("ssm_conv_silu(Tensor u, Tensor w, Tensor b, Tensor(a!) state, Tensor cu, Tensor seq_of, Tensor slots, Tensor pos, "
-        "bool single) -> Tensor");
+  m.def("ssm_conv_silu(Tensor u, Tensor w, Tensor? b, Tensor(a!) state, Tensor cu, Tensor seq_of, Tensor slots, Tensor pos, "
+        "bool single, bool act) -> Tensor");
   m.def("ssm_selective_scan(Tensor x, Tensor Bm, Tensor Cm, Tensor dt, Tensor dt_bias, Tensor a_log, Tensor d_skip, "
         "Tensor(a!) S, Tensor cu, Tensor slots, Tensor pos) -> Tensor");
   m.def("ssm_gated_group_norm(Tensor y, Tensor z, Tensor w, int groups, float eps, bool act_f32) -> Tensor");

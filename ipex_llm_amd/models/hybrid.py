@@ -490,8 +490,9 @@ class MaskedAttention(nn.Module):
         """``y``: this mixer's columns of the input projection, ``[q | k | v | gate]``"""
         s = self.s
         T, H, G, d, dv = y.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        act = y.dtype
         gate = y[:, self.n_qkv:] if s.out_gate else None
-        if self.conv is not None:
+        if self.conv is not None:               # f32 result: the norm and the rotation read it unrounded
             y = GM.causal_conv(y[:, :self.n_qkv], self.conv, cache.state[li]["conv"], meta.cu_q, meta.seq_of,
                                meta.state_slots, pos, meta.q_lens_host)
         q = y[:, :H * d].view(T, H, d)
@@ -508,7 +509,7 @@ class MaskedAttention(nn.Module):
             qf = MA.qkv_norm_rope_store(q, None, None, self.q_norm, None, s.qk_norm == "whole", eps, table,
                                         layout, pos, slots, None)
         o = MA.masked_attention(qf, rows, G, dv, meta.block_tables, meta.seq_of, pos, s.scale, s.mask.kind, s.mask.size,
-                                self.sink, meta.q_lens_host, meta.seq_lens_host, y.dtype, softcap=s.softcap,
+                                self.sink, meta.q_lens_host, meta.seq_lens_host, act, softcap=s.softcap,
                                 keep_first=s.mask.keep_first, talk=self.talk)
         if gate is not None:
             o = MA.sigmoid_gate(o, gate)

@@ -73,7 +73,8 @@ def require_seqmix():
         full = os.path.exists(_LIB_PATH)
     if full:
         lib = require()
-        if not hasattr(lib, "sm_latent_attention") or not hasattr(lib, "bm_talk_attention"):
+        if not hasattr(lib, "sm_latent_attention") or not hasattr(lib, "bm_talk_attention") or \
+                not hasattr(lib, "gm_gla_scan"):
             raise RuntimeError(f"{_LIB_PATH} predates the sequence-mixing kernels: rebuild it "
                                "(python -m ipex_llm_amd._build)")
         return lib

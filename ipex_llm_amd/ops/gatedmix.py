@@ -22,6 +22,7 @@ import torch
 import torch.nn.functional as F
 
 from .seqmix import native
+from .ssm import conv_silu
 
 __all__ = ["layer_norm_pair_shift", "causal_conv", "mingru_scan", "gla_scan", "head_rms_silu", "rms_pair_mean",
            "softcap_", "GLA_MAX_DIM"]
@@ -76,41 +77,13 @@ def layer_norm_pair_shift(x: torch.Tensor, w1: torch.Tensor, w2: Optional[torch.
 
 def causal_conv(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu: torch.Tensor, seq_of: torch.Tensor,
                 state_slots: torch.Tensor, pos: torch.Tensor, q_lens: List[int]) -> torch.Tensor:
-    """Causal per-channel convolution over time, no bias, no activation.
+    """Causal per-channel convolution over time, no bias, no activation: the
+    convolution of ``ops/ssm.py`` (same kernel, same state layout) without its
+    bias and SiLU.  ``u`` [T, C], ``w`` f32 [C, taps], ``state`` f32
+    [slots, taps - 1, C]:
 
-    ``u`` [T, C] (a strided view of a projection's result is allowed), ``w``
-    f32 [C, taps] whose last column weighs the current token:
-
-        out_t = sum_j w[:, j] * u_(t - taps + 1 + j)                 [T, C] in u's dtype
-
-    with zeros before a sequence's start and f32 accumulation.  ``state`` f32
-    [slots, taps - 1, C] holds, per sequence, the inputs of its last
-    ``taps - 1`` positions (oldest first); a portion that does not start at
-    position 0 reads what lies before it from there, and every portion leaves
-    its last inputs there."""
-    taps = w.shape[1]
-    if native(u):
-        return _ops().gm_causal_conv(u, w, state, cu, seq_of, state_slots, pos, _single(q_lens, u.shape[0]))
-    T, C = u.shape
-    out = torch.empty(T, C, dtype=u.dtype, device=u.device)
-    uf = u.float()
-    slots, first = state_slots.tolist(), pos.tolist()
-    t0 = 0
-    for s, n in enumerate(q_lens):
-        if n == 0:
-            continue
-        p0 = first[t0]
-        hist = state[slots[s]].clone()                              # positions p0 - taps + 1 .. p0 - 1
-        if p0 < taps - 1:
-            hist[:taps - 1 - p0] = 0.0
-        ext = torch.cat([hist, uf[t0:t0 + n]], 0)
-        acc = torch.zeros(n, C, dtype=torch.float32, device=u.device)
-        for j in range(taps):
-            acc += w[:, j].float()[None] * ext[j:j + n]
-        out[t0:t0 + n] = acc.to(u.dtype)
-        state[slots[s]] = ext[n:]
-        t0 += n
-    return out
+        out_t = sum_j w[:, j] * u_(t - taps + 1 + j)                 f32 [T, C]"""
+    return conv_silu(u, w, None, state, cu, seq_of, state_slots, pos, q_lens, act=False)
 
 
 def mingru_scan(y: torch.Tensor, width: int, state: torch.Tensor, cu: torch.Tensor, state_slots: torch.Tensor,
@@ -128,7 +101,7 @@ def mingru_scan(y: torch.Tensor, width: int, state: torch.Tensor, cu: torch.Tens
     after the last token.  Returns [T, width] in y's dtype."""
     T = y.shape[0]
     if native(y):
-        return _ops().gm_mingru_scan(y, width, state, cu, state_slots, pos)
+        return _ops().gm_mingru_scan(y, width, state, cu, state_slots, pos, max(q_lens))
     yf = y.float()
     z = torch.sigmoid(yf[:, :width])
     u = yf[:, width:2 * width]

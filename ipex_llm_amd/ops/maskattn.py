@@ -164,7 +164,7 @@ def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block
     return out.reshape(T, H * dv).to(out_dtype)
 
 
-def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out):
+def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out, softcap=0.0, talk=None):
     """``nc`` pieces of chunks of one sequence: piece i holds the ``nk`` keys from position ``lo + i nk`` (a chunk's
     first position) on, and its queries are its last ``nq`` positions (whole chunks: nq == nk == the chunk size;
     one piece with nq < nk: a portion that starts inside a chunk); the step's token ``t0`` is the first query.
@@ -183,7 +183,9 @@ def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out
     qq = q[t0:t0 + n].view(nc, nq, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, nq * rep, d)
     if f32:
         sc = torch.bmm(qq, kk)
-        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, True)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, True, softcap, True)
+        if talk is not None:
+            w = _ops().ma_talk_mix(w, talk, nq, G, rep, True)
         o = torch.bmm(w.view(nc * G, nq * rep, nk), vv)
     else:
         # f32 queries against 16-bit keys, f32 weights against 16-bit values: hi + lo halves side by side along the
@@ -191,22 +193,27 @@ def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out
         qh = qq.to(rows.dtype)
         q2 = torch.cat([qh, (qq - qh.float()).to(rows.dtype)], -1)
         sc = torch.bmm(q2, torch.cat([kk, kk], 1), out_dtype=torch.float32)
-        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False)
+        if talk is None:
+            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, False)
+        else:       # normalised f32 weights in place, then the heads' weights mixed and split into hi + lo halves
+            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, True)
+            w = _ops().ma_talk_mix(w, talk, nq, G, rep, False)
         o = torch.bmm(w.view(nc * G, nq * rep, 2 * nk), torch.cat([vv, vv], 1), out_dtype=torch.float32)
     o = o.view(nc, G, nq, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
     out[t0:t0 + n] = o.to(out.dtype)
 
 
 def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask, size, sink, q_lens, ctx_lens,
-                          out_dtype):
+                          out_dtype, softcap=0.0, keep_first=0, talk=None):
     T, H, d = q.shape
     f32 = out_dtype == torch.float32
     q = q.contiguous()
     code = MASKS[mask]
-    big = mask == "chunk" and GEMM_MIN_CHUNK > 0 and max(q_lens) >= GEMM_MIN_CHUNK and _bmm_f32_ok(rows.dtype)
+    big = mask == "chunk" and GEMM_MIN_CHUNK > 0 and max(q_lens) >= GEMM_MIN_CHUNK and _bmm_f32_ok(rows.dtype) and \
+        (talk is None or H <= 256)
     if not big:
         return _ops().ma_masked_attention(q, rows, G, dv, block_tables, seq_of, pos, scale, code, size, sink,
-                                          max(ctx_lens), f32)
+                                          max(ctx_lens), f32, softcap, keep_first, talk)
     out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
     rest, rest_ctx, t0 = [], 1, 0
     for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
@@ -222,7 +229,7 @@ def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask
                 nc, nq = 1, min(L, c0 + size) - p0
                 nk = p0 - c0 + nq
             if nq >= GEMM_MIN_CHUNK:
-                _pieces_gemm(q, rows, block_tables[b], G, dv, scale, sink, t, c0, nc, nk, nq, out)
+                _pieces_gemm(q, rows, block_tables[b], G, dv, scale, sink, t, c0, nc, nk, nq, out, softcap, talk)
             else:
                 rest.append(torch.arange(t, t + nc * nq, device=q.device))
                 rest_ctx = max(rest_ctx, L)
@@ -232,7 +239,8 @@ def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask
     if rest:
         idx = torch.cat(rest)
         out[idx] = _ops().ma_masked_attention(q[idx].contiguous(), rows, G, dv, block_tables, seq_of[idx].contiguous(),
-                                              pos[idx].contiguous(), scale, code, size, sink, rest_ctx, f32)
+                                              pos[idx].contiguous(), scale, code, size, sink, rest_ctx, f32, softcap,
+                                              keep_first, talk)
     return out
 
 

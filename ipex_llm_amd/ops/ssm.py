@@ -14,7 +14,7 @@ and accumulates in f32, and its result stays f32 for the scan.
 """
 from __future__ import annotations
 
-from typing import List
+from typing import List, Optional
 
 import torch
 import torch.nn.functional as F
@@ -30,9 +30,10 @@ def _ops():
     return torch.ops.ipex_llm_amd
 
 
-def conv_silu(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor, state: torch.Tensor, cu: torch.Tensor,
-              seq_of: torch.Tensor, state_slots: torch.Tensor, pos: torch.Tensor, q_lens: List[int]) -> torch.Tensor:
-    """Causal per-channel convolution over time with bias, then SiLU.
+def conv_silu(u: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], state: torch.Tensor, cu: torch.Tensor,
+              seq_of: torch.Tensor, state_slots: torch.Tensor, pos: torch.Tensor, q_lens: List[int],
+              act: bool = True) -> torch.Tensor:
+    """Causal per-channel convolution over time with bias (``b`` None: none), then SiLU (``act`` False: none).
 
     ``u`` [T, C] (a strided view of a projection's result is allowed), ``w``
     f32 [C, taps] whose last column weighs the current token, ``b`` f32 [C]:
@@ -46,7 +47,7 @@ def conv_silu(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor, state: torch.Te
     taps = w.shape[1]
     if native(u):
         single = len(q_lens) == u.shape[0] and all(n == 1 for n in q_lens)
-        return _ops().ssm_conv_silu(u, w, b, state, cu, seq_of, state_slots, pos, single)
+        return _ops().ssm_conv_silu(u, w, b, state, cu, seq_of, state_slots, pos, single, act)
     T, C = u.shape
     out = torch.empty(T, C, dtype=torch.float32, device=u.device)
     uf = u.float()
@@ -60,10 +61,10 @@ def conv_silu(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor, state: torch.Te
         if p0 < taps - 1:
             hist[:taps - 1 - p0] = 0.0
         ext = torch.cat([hist, uf[t0:t0 + n]], 0)
-        acc = b.float()[None].repeat(n, 1)
+        acc = b.float()[None].repeat(n, 1) if b is not None else torch.zeros(n, C, device=u.device)
         for j in range(taps):
             acc += w[:, j].float()[None] * ext[j:j + n]
-        out[t0:t0 + n] = F.silu(acc)
+        out[t0:t0 + n] = F.silu(acc) if act else acc
         state[slots[s]] = ext[n:]
         t0 += n
     return out

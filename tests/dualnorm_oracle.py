@@ -130,10 +130,8 @@ def window_attention(W, p, m, h):
         g = hd // (H // G)
         for i in range(T):
             js = [j for j in range(i + 1) if visible(i, j, m["mask"], False)]
-            s = torch.stack([(q[i, hd] * k[j, g]).sum() * float(m["scale"]) for j in js])
-            w = torch.softmax(s, 0)
-            for wj, j in zip(w, js):
-                out[i, hd] += wj * v[j, g]
+            s = (k[js, g] @ q[i, hd]) * float(m["scale"])
+            out[i, hd] = torch.softmax(s, 0) @ v[js, g]
     o = out.reshape(T, H * dv) * sigmoid(h @ W[p + "g"].T)
     return o @ W[p + "o"].T
 
@@ -183,7 +181,7 @@ def chunk_attention(W, p, m, h, eps, kv):
         g = hd // (H // G)
         for i in range(T):
             js = [j for j in range(i + 1) if visible(i, j, m["mask"], True)]
-            s = torch.stack([(q[i, hd] * k[j, g]).sum() * float(m["scale"]) for j in js])
+            s = (k[js, g] @ q[i, hd]) * float(m["scale"])
             if cap:
                 s = cap * torch.tanh(s / cap)
             e = torch.exp(s)
