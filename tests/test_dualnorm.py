@@ -286,7 +286,7 @@ def test_router_and_experts(dev):
         z = torch.randn(T, E, generator=g) * 3
         z[0, :] = 1.5                                                 # all equal: the first `top` indices
         idx, wts = BM.moe_route(z.to(dev), top, "softmax")
-        order = torch.sort(z.double(), -1, descending=True, stable=True)
+        order = torch.sort(z.double(), dim=-1, descending=True, stable=True)
         assert torch.equal(idx.cpu().long(), order.indices[:, :top])
         assert (wts.double().cpu() - torch.softmax(order.values[:, :top], -1)).abs().max() < 1e-6
         for act in (torch.float32, torch.bfloat16):
