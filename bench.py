@@ -178,7 +178,19 @@ def main():
     ap.add_argument("--prenorm-sizes", default="small,base")
     ap.add_argument("--prenorm-prompts", default="1024,4096")
     ap.add_argument("--no-prenorm-ref", action="store_true", help="--prenorm: skip the comparison model")
+    ap.add_argument("--twonorm", action="store_true",
+                    help="side benchmark (not the headline metric): prefill / decode throughput of the decoder of "
+                         "two-norm parallel blocks (chunked attention with mixed head weights, minGRU, windowed attention "
+                         "beside gated linear attention, softmax-routed experts) beside the parallel-residual decoder "
+                         "with experts at equal sizes, one GPU")
+    ap.add_argument("--twonorm-sizes", default="small,base")
+    ap.add_argument("--twonorm-prompts", default="1024,4096")
+    ap.add_argument("--no-twonorm-ref", action="store_true", help="--twonorm: skip the comparison model")
     args = ap.parse_args()
+    if args.twonorm:
+        from ipex_llm_amd.utils.bench_twonorm import main as twonorm_main
+        twonorm_main(args)
+        return
     if args.prenorm:
         from ipex_llm_amd.utils.bench_prenorm import main as prenorm_main
         prenorm_main(args)

@@ -153,14 +153,25 @@ __global__ void __launch_bounds__(1024) mingru_scan_k(const E* __restrict__ y, i
   const E* yz = y + (int64_t)t0 * y_ld + (ok ? c : 0);
   // the piece folded: S_out = A S_in + B
   float A = 1.f, Bv = 0.f;
+  constexpr int UN = 8;                                             // tokens whose inputs are requested together
   if (NC > 1) {
     if (ok)
-      for (int t = lo; t < hi; t++) {
-        const float z = sigmoidf(ldf(yz + (int64_t)t * y_ld));
-        const float u = ldf(yz + (int64_t)t * y_ld + width);
-        const float cand = u >= 0.f ? u + 0.5f : sigmoidf(u);
-        A *= 1.0f - z;
-        Bv = fmaf(1.0f - z, Bv, z * cand);
+      for (int tb = lo; tb < hi; tb += UN) {
+        float zr[UN], ur[UN];
+#pragma unroll
+        for (int i = 0; i < UN; i++) {
+          const int t = min(tb + i, hi - 1);
+          zr[i] = ldf(yz + (int64_t)t * y_ld);
+          ur[i] = ldf(yz + (int64_t)t * y_ld + width);
+        }
+#pragma unroll
+        for (int i = 0; i < UN; i++) {
+          if (tb + i >= hi) break;
+          const float z = sigmoidf(zr[i]);
+          const float cand = ur[i] >= 0.f ? ur[i] + 0.5f : sigmoidf(ur[i]);
+          A *= 1.0f - z;
+          Bv = fmaf(1.0f - z, Bv, z * cand);
+        }
       }
     fa[j][lane] = A;
     fb[j][lane] = Bv;
@@ -172,20 +183,31 @@ __global__ void __launch_bounds__(1024) mingru_scan_k(const E* __restrict__ y, i
   __syncthreads();                                                  // every piece has read the slot
   if (!ok) return;
   E* o = out + (int64_t)t0 * width + c;
-  for (int t = lo; t < hi; t++) {
-    const float z = sigmoidf(ldf(yz + (int64_t)t * y_ld));
-    const float u = ldf(yz + (int64_t)t * y_ld + width);
-    const float g = ldf(yz + (int64_t)t * y_ld + 2 * width);
-    const float cand = u >= 0.f ? u + 0.5f : sigmoidf(u);
-    S = fmaf(1.0f - z, S, z * cand);
-    stf(o + (int64_t)t * width, S * silu(g));
+  for (int tb = lo; tb < hi; tb += UN) {
+    float zr[UN], ur[UN], gr[UN];
+#pragma unroll
+    for (int i = 0; i < UN; i++) {
+      const int t = min(tb + i, hi - 1);
+      zr[i] = ldf(yz + (int64_t)t * y_ld);
+      ur[i] = ldf(yz + (int64_t)t * y_ld + width);
+      gr[i] = ldf(yz + (int64_t)t * y_ld + 2 * width);
+    }
+#pragma unroll
+    for (int i = 0; i < UN; i++) {
+      if (tb + i >= hi) break;
+      const float z = sigmoidf(zr[i]);
+      const float cand = ur[i] >= 0.f ? ur[i] + 0.5f : sigmoidf(ur[i]);
+      S = fmaf(1.0f - z, S, z * cand);
+      stf(o + (int64_t)(tb + i) * width, S * silu(gr[i]));
+    }
   }
   if (hi == n && lo < n) *st = S;                                   // the piece that holds the last token
 }
 
 // ------------------------------------------------------------------ gated linear attention
-template <typename E, int NS>
-__global__ void __launch_bounds__(1024) gla_scan_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
+// MAXT: the most threads a launch brings (256, 512 or 1024: the register budget follows it)
+template <typename E, int NS, int MAXT>
+__global__ void __launch_bounds__(MAXT) gla_scan_k(const E* __restrict__ q, int64_t q_ld, const E* __restrict__ k,
                                                   int64_t k_ld, const E* __restrict__ v, int64_t v_ld,
                                                   const E* __restrict__ a, int64_t a_ld, float inv_tau, float q_scale,
                                                   float* __restrict__ S, const int32_t* __restrict__ cu,
@@ -347,7 +369,7 @@ void gla_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_l
   int NS = 64;
   for (int ns = 8; ns <= 64; ns *= 2) {
     const int nw = (d + ns - 1) / ns;
-    if (nw <= 16 && (ns == 64 || cols * ((d + 2 * ns - 1) / (2 * ns)) < 2048)) {
+    if (nw <= 16 && (ns == 64 || cols * ((d + 2 * ns - 1) / (2 * ns)) < 1024)) {
       NS = ns;
       break;
     }
@@ -358,17 +380,23 @@ void gla_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_l
   TC = TC > 32 ? 32 : (TC < 1 ? 1 : TC);
   const size_t lds = per_tok * TC;
   const dim3 grid(B, H, (dv + 63) / 64), block(64 * NW);
-#define GM_GLA(E, NSV)                                                                                          \
-  gla_scan_k<E, NSV><<<grid, block, lds, st>>>((const E*)q, q_ld, (const E*)k, k_ld, (const E*)v, v_ld, (const E*)a, \
-                                               a_ld, 1.0f / tau, q_scale, S, cu, slots, pos, out, H, d, dv, TC)
+#define GM_GLA_T(E, NSV, MT)                                                                                        \
+  gla_scan_k<E, NSV, MT><<<grid, block, lds, st>>>((const E*)q, q_ld, (const E*)k, k_ld, (const E*)v, v_ld,          \
+                                                   (const E*)a, a_ld, 1.0f / tau, q_scale, S, cu, slots, pos, out, H, \
+                                                   d, dv, TC)
+#define GM_GLA(E, NSV)                          \
+  if (NW <= 4) GM_GLA_T(E, NSV, 256);           \
+  else if (NW <= 8) GM_GLA_T(E, NSV, 512);      \
+  else GM_GLA_T(E, NSV, 1024)
 #define GM_GLA_NS(E)                     \
-  if (NS == 8) GM_GLA(E, 8);             \
-  else if (NS == 16) GM_GLA(E, 16);      \
-  else if (NS == 32) GM_GLA(E, 32);      \
-  else GM_GLA(E, 64)
+  if (NS == 8) { GM_GLA(E, 8); }         \
+  else if (NS == 16) { GM_GLA(E, 16); }  \
+  else if (NS == 32) { GM_GLA(E, 32); }  \
+  else { GM_GLA(E, 64); }
   if (bf16) { GM_GLA_NS(__bf16); } else { GM_GLA_NS(float); }
 #undef GM_GLA_NS
 #undef GM_GLA
+#undef GM_GLA_T
 }
 
 void head_rms_silu(bool bf16, const float* o, const void* w, const void* gate, int64_t g_ld, void* out, int T, int H,

@@ -40,9 +40,11 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
 // its last Lq positions (Lq == L: a whole chunk).  Row i: head (i / (rep Lq)) % G * rep + i % rep, query
 // (i / rep) % Lq, which sees keys 0 .. L - Lq + query.  Scaled, softmax with the head's sink; bf16: the f32 weights
 // leave as bf16 pairs hi + lo in hl [R, 2 L] (a row's hi halves, then its lo halves); f32 (hl == null): in place
-// (hl null with bf16: in place as well); softcap as above
+// (hl null with bf16: in place as well); softcap as above.  window > 0: the rows are a block of Lq queries of a sliding
+// window instead (query i at position q0 + i): the first nkeep columns are kept first tokens, column nkeep + j is the
+// key at position k0 + j, seen when not ahead of the query and closer than ``window`` (or before position ``keep``)
 void chunk_softmax(bool bf16, float* sc, int64_t R, int Lq, int L, int G, int rep, float scale, const float* sink,
-                   void* hl, float softcap, hipStream_t st);
+                   void* hl, float softcap, int window, int keep, int nkeep, int64_t q0, int64_t k0, hipStream_t st);
 
 // w f32 [pieces, G, Lq, rep, L] normalised weights -> the heads' weights mixed by talk f32 [H, H] (H = G rep), same
 // layout: bf16 pairs hi + lo in hl [R, 2 L], or f32 in out32 [R, L]

@@ -381,26 +381,28 @@ __global__ void __launch_bounds__(64) masked_attn_combine_k(const float* __restr
 // part [T, H, G, nsplit, dv + 2] holds, for query head g and value head c, the unnormalised sums of every key split.
 // One wave per (token, output head); dv <= 512
 template <typename E>
-__global__ void __launch_bounds__(64) masked_attn_talk_combine_k(const float* __restrict__ part,
-                                                                const float* __restrict__ sink,
-                                                                const float* __restrict__ talk, E* __restrict__ out,
-                                                                int H, int G, int dv, int nsplit) {
-  __shared__ float wz[64];
+__global__ void __launch_bounds__(512) masked_attn_talk_combine_k(const float* __restrict__ part,
+                                                                 const float* __restrict__ sink,
+                                                                 const float* __restrict__ talk, E* __restrict__ out,
+                                                                 int H, int G, int dv, int nsplit) {
+  extern __shared__ float cs[];                                     // [NW][64] split factors, then [NW][dv] sums
   const int64_t t = blockIdx.x;
-  const int h = blockIdx.y, c = h / (H / G), lane = threadIdx.x;
+  const int h = blockIdx.y, c = h / (H / G), lane = threadIdx.x & 63, wv = threadIdx.x >> 6, NW = blockDim.x >> 6;
+  float* wz = cs + wv * 64;
+  float* sums = cs + NW * 64;
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = 0.f;
-  for (int g = 0; g < H; g++) {
+  for (int g = wv; g < H; g += NW) {                                // wave w: source heads w, w + NW, ...
     const float* pp = part + ((t * H + g) * G + c) * (int64_t)nsplit * (dv + 2);
     const float mz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv] : -INFINITY;
     const float lz = lane < nsplit ? pp[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
     const float sk = sink ? sink[g] : -INFINITY;
     const float M = fmaxf(wave_max(mz), sk);
     const float f = mz == -INFINITY ? 0.f : expf(mz - M);
-    __syncthreads();
+    wave_sync();
     wz[lane] = f;
-    __syncthreads();
+    wave_sync();
     float L = sink ? expf(sk - M) : 0.f;
     for (int z = 0; z < nsplit; z++) L += __shfl(lz, z, 64) * wz[z];   // index order, whatever the lanes do
     const float coef = talk[h * H + g] / L;
@@ -417,7 +419,13 @@ __global__ void __launch_bounds__(64) masked_attn_talk_combine_k(const float* __
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const int col = lane + 64 * i;
-    if (col < dv) stf(out + (t * H + h) * dv + col, acc[i]);
+    if (col < dv) sums[wv * dv + col] = acc[i];
+  }
+  __syncthreads();
+  for (int col = threadIdx.x; col < dv; col += blockDim.x) {
+    float o = 0.f;
+    for (int w = 0; w < NW; w++) o += sums[w * dv + col];           // the waves in order
+    stf(out + (t * H + h) * dv + col, o);
   }
 }
 
@@ -453,20 +461,30 @@ __global__ void __launch_bounds__(64) talk_mix_k(const float* __restrict__ w, co
 }
 
 // ------------------------------------------------------------------ softmax between the chunk products
+// window == 0: a piece of a chunk (query tok sees keys 0 .. L - Lq + tok).  window > 0: a block of queries of a
+// sliding window: query tok stands at position q0 + tok; the first nkeep columns are kept first tokens (always
+// visible), column nkeep + jj is the key at position k0 + jj, visible when it is not ahead of the query and inside
+// the window (or before position ``keep``)
 template <typename E>
 __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, int Lq, int L, int G, int rep, float scale,
-                                                      const float* __restrict__ sink, E* __restrict__ hi, float softcap) {
+                                                      const float* __restrict__ sink, E* __restrict__ hi, float softcap,
+                                                      int window, int keep, int nkeep, int64_t q0, int64_t k0) {
   __shared__ float red[16];
   const int64_t row = blockIdx.x;
   const int tok = (int)((row / rep) % Lq);                          // the piece's queries are its last Lq positions
   const int h = (int)((row / ((int64_t)rep * Lq)) % G) * rep + (int)(row % rep);
-  const int nk = L - Lq + tok + 1;
+  const int64_t p = q0 + tok;
+  const int nk = window > 0 ? (int)min((int64_t)L, nkeep + (p - k0) + 1) : L - Lq + tok + 1;
+  // the first column of the window's own keys (columns nkeep .. first - 1 are seen only if kept)
+  const int first = window > 0 ? nkeep + (int)max((int64_t)0, p - window + 1 - k0) : 0;
+  auto vis = [&](int j) -> bool { return window <= 0 || j < nkeep || j >= first || k0 + (j - nkeep) < keep; };
   float* s = sc + row * L;
   const float sk = sink ? sink[h] : -INFINITY;
   float mx = sk;
   for (int j = threadIdx.x; j < nk; j += blockDim.x) {
     float v = s[j] * scale;
     if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+    if (!vis(j)) v = -INFINITY;
     s[j] = v;
     mx = fmaxf(mx, v);
   }
@@ -477,7 +495,7 @@ __global__ void __launch_bounds__(256) chunk_softmax_k(float* __restrict__ sc, i
   for (int i = 0; i < (int)(blockDim.x >> 6); i++) mx = fmaxf(mx, red[i]);
   float sum = 0.f;
   for (int j = threadIdx.x; j < nk; j += blockDim.x) {
-    const float e = expf(s[j] - mx);
+    const float e = expf(s[j] - mx);                               // a masked column: exp(-inf) = 0
     s[j] = e;
     sum += e;
   }
@@ -596,8 +614,12 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
 #undef MA_RC
 #undef MA_LAUNCH
   if (cross) {
-    if (bf16) masked_attn_talk_combine_k<__bf16><<<dim3(T, H), 64, 0, st>>>(part, sink, talk, (__bf16*)out, H, G, dv, nsplit);
-    else masked_attn_talk_combine_k<float><<<dim3(T, H), 64, 0, st>>>(part, sink, talk, (float*)out, H, G, dv, nsplit);
+    const int cw = H < 8 ? H : 8;                                   // waves: each merges some of the source heads
+    const size_t cl = (size_t)cw * (64 + dv) * sizeof(float);
+    if (bf16)
+      masked_attn_talk_combine_k<__bf16><<<dim3(T, H), 64 * cw, cl, st>>>(part, sink, talk, (__bf16*)out, H, G, dv, nsplit);
+    else
+      masked_attn_talk_combine_k<float><<<dim3(T, H), 64 * cw, cl, st>>>(part, sink, talk, (float*)out, H, G, dv, nsplit);
   } else if (nsplit > 1) {
     if (bf16) masked_attn_combine_k<__bf16><<<dim3(T, H), 64, 0, st>>>(part, sink, (__bf16*)out, H, dv, nsplit);
     else masked_attn_combine_k<float><<<dim3(T, H), 64, 0, st>>>(part, sink, (float*)out, H, dv, nsplit);
@@ -605,10 +627,14 @@ void masked_attention(bool bf16, const float* q, const void* rows, int bs, const
 }
 
 void chunk_softmax(bool bf16, float* sc, int64_t R, int Lq, int L, int G, int rep, float scale, const float* sink,
-                   void* hl, float softcap, hipStream_t st) {
+                   void* hl, float softcap, int window, int keep, int nkeep, int64_t q0, int64_t k0, hipStream_t st) {
   if (R <= 0 || L <= 0) return;
-  if (bf16) chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (__bf16*)hl, softcap);
-  else chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (float*)nullptr, softcap);
+  if (bf16)
+    chunk_softmax_k<__bf16><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (__bf16*)hl, softcap, window,
+                                                         keep, nkeep, q0, k0);
+  else
+    chunk_softmax_k<float><<<(unsigned)R, 256, 0, st>>>(sc, Lq, L, G, rep, scale, sink, (float*)nullptr, softcap, window,
+                                                        keep, nkeep, q0, k0);
 }
 
 void talk_mix(bool bf16, const float* w, const float* talk, int64_t pieces, int Lq, int L, int G, int rep, void* hl,

@@ -145,13 +145,17 @@ int64_t ma_masked_attention_fits(bool bf16, int64_t rep, int64_t d, int64_t dv) 
 // scores f32 [R, L] of whole chunks -> softmax weights with the sink: bf16 [R, 2 L] (hi halves | lo halves), or in
 // place (f32)
 Tensor ma_chunk_softmax(Tensor& scores, int64_t Lq, int64_t G, int64_t rep, double scale,
-                        const c10::optional<Tensor>& sink, bool act_f32, double softcap, bool in_place) {
+                        const c10::optional<Tensor>& sink, bool act_f32, double softcap, bool in_place, int64_t window,
+                        int64_t keep, int64_t nkeep, int64_t q0, int64_t k0) {
   c10::DeviceGuard g(scores.device());
   TORCH_CHECK(scores.is_cuda() && scores.dim() == 2 && scores.scalar_type() == at::kFloat && scores.is_contiguous(),
               "ma_chunk_softmax: scores f32 [R, L] contiguous");
   const int64_t R = scores.size(0), L = scores.size(1);
-  TORCH_CHECK(G >= 1 && rep >= 1 && Lq >= 1 && Lq <= L && R % (G * rep * Lq) == 0,
+  TORCH_CHECK(G >= 1 && rep >= 1 && Lq >= 1 && (window > 0 || Lq <= L) && R % (G * rep * Lq) == 0,
               "ma_chunk_softmax: rows must be pieces x key heads x Lq x rep, Lq <= L");
+  TORCH_CHECK(window >= 0 && window < (int64_t)1 << 30 && keep >= 0 && keep < (int64_t)1 << 30 && nkeep >= 0 &&
+                  nkeep <= L && q0 >= 0 && k0 >= 0 && k0 <= q0 && (window == 0 || nkeep + (q0 - k0) + Lq <= L),
+              "ma_chunk_softmax: a window's block holds its kept columns and every key from k0 to its last query");
   const float* sk = nullptr;
   if (has(sink)) {
     TORCH_CHECK(sink->is_cuda() && sink->scalar_type() == at::kFloat && sink->is_contiguous() && sink->numel() == G * rep,
@@ -162,7 +166,8 @@ Tensor ma_chunk_softmax(Tensor& scores, int64_t Lq, int64_t G, int64_t rep, doub
   const bool pairs = !act_f32 && !in_place;
   if (pairs) hl = at::empty({R, 2 * L}, scores.options().dtype(at::kBFloat16));
   illm::ma::chunk_softmax(!act_f32, scores.data_ptr<float>(), R, (int)Lq, (int)L, (int)G, (int)rep, (float)scale, sk,
-                          pairs ? hl.data_ptr() : nullptr, (float)softcap, stream());
+                          pairs ? hl.data_ptr() : nullptr, (float)softcap, (int)window, (int)keep, (int)nkeep, q0, k0,
+                          stream());
   return pairs ? hl : scores;
 }
 
@@ -205,7 +210,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
         "Tensor? talk) -> Tensor");
   m.def("ma_masked_attention_fits(bool bf16, int rep, int d, int dv) -> int");
   m.def("ma_chunk_softmax(Tensor(a!) scores, int Lq, int G, int rep, float scale, Tensor? sink, bool act_f32, "
-        "float softcap, bool in_place) -> Tensor");
+        "float softcap, bool in_place, int window, int keep, int nkeep, int q0, int k0) -> Tensor");
   m.def("ma_talk_mix(Tensor w, Tensor talk, int Lq, int G, int rep, bool act_f32) -> Tensor");
   m.def("ma_sigmoid_gate(Tensor(a!) o, Tensor gate) -> Tensor(a!)");
 }

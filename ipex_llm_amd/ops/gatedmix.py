@@ -16,6 +16,7 @@ whatever the activation dtype is; the convolution accumulates in f32.
 """
 from __future__ import annotations
 
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -142,6 +143,8 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_pre: torch.Ten
     if native(q):
         if d > GLA_MAX_DIM:
             raise ValueError(f"gla_scan: key size {d} is above the kernel's {GLA_MAX_DIM}")
+        if GLA_PIECE_MIN > 0 and max(q_lens) >= GLA_PIECE_MIN:
+            return _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_lens)
         return _ops().gm_gla_scan(q, k, v, a_pre, tau, q_scale, state, cu, state_slots, pos)
     out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
     alpha = torch.exp(F.logsigmoid(a_pre.float()) / tau)
@@ -157,6 +160,63 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_pre: torch.Ten
             out[t] = torch.einsum("hdp,hd->hp", S, qf[t])
         state[slots[s]] = S
         t0 += n
+    return out
+
+
+# The scan is sequential in time.  A portion of at least GLA_PIECE_MIN tokens is cut into up to GLA_PIECES pieces
+# that run side by side, twice: the recurrence is linear in the state, S_end = diag(P) S_start + Z with P the product
+# of the piece's decays and Z its result from a zero state, so a first pass gives every piece's Z, a short chain
+# over the pieces gives every piece's true start state, and a second pass from those writes the outputs.
+GLA_PIECE_MIN = int(os.environ.get("ILLM_GLA_PIECE_MIN", "1024"))
+GLA_PIECES = int(os.environ.get("ILLM_GLA_PIECES", "16"))
+
+
+def _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_lens):
+    T, H, d = q.shape
+    dev = q.device
+    cuts, first, owner, spans = [0], [], [], []      # piece borders (token indices); first piece of / pieces per sequence
+    t0 = 0
+    for s, n in enumerate(q_lens):
+        if n == 0:
+            continue
+        per = max(-(-n // GLA_PIECES), 64) if n >= GLA_PIECE_MIN else n
+        first.append(len(cuts) - 1)
+        for lo in range(0, n, per):
+            cuts.append(t0 + min(n, lo + per))
+        owner.append((s, len(cuts) - 1 - first[-1]))
+        spans.append((t0, n, per))
+        t0 += n
+    NP = len(cuts) - 1
+    cu_p = torch.tensor(cuts, dtype=torch.int32, device=dev)
+    slots_p = torch.arange(NP, dtype=torch.int32, device=dev)
+    first_t = torch.tensor(first, dtype=torch.long, device=dev)
+    seqs = torch.tensor([s for s, _ in owner], dtype=torch.long, device=dev)
+    real = state_slots.long().index_select(0, seqs)
+    later = torch.tensor([cuts[f + j] for f, (_, m) in zip(first, owner) for j in range(1, m)], dtype=torch.long, device=dev)
+    # every piece's decay product (of the sequences that have several pieces): sums of log decays in f64
+    P = {}
+    for f, (_, m), (s0, n, per) in zip(first, owner, spans):
+        if m > 1:
+            ls = F.logsigmoid(a_pre[s0:s0 + n].float())
+            ls = F.pad(ls, (0, 0, 0, 0, 0, m * per - n)).view(m, per, H, d).double().sum(1)
+            P[f] = torch.exp(ls / tau).float()                          # [m, H, d]
+    start = state.index_select(0, real)
+    Z = torch.empty(NP + 1, *state.shape[1:], dtype=torch.float32, device=dev)
+    Z.index_copy_(0, first_t, start)
+    pos1 = pos.clone()
+    pos1.index_fill_(0, later, 0)                                       # later pieces start from zero in the first pass
+    _ops().gm_gla_scan(q, k, v, a_pre, tau, q_scale, Z, cu_p, slots_p, pos1)
+    Sin = torch.empty_like(Z)
+    Sin.index_copy_(0, first_t, start)
+    for f, (_, m) in zip(first, owner):                                 # the chain of start states, piece after piece
+        for j in range(1, m):
+            if j == 1:
+                Sin[f + 1].copy_(Z[f])                                  # the first piece's Z holds its start state too
+            else:
+                torch.addcmul(Z[f + j - 1], Sin[f + j - 1], P[f][j - 1].unsqueeze(-1), out=Sin[f + j])
+    out = _ops().gm_gla_scan(q, k, v, a_pre, tau, q_scale, Sin, cu_p, slots_p, pos)
+    last = torch.tensor([f + m - 1 for f, (_, m) in zip(first, owner)], dtype=torch.long, device=dev)
+    state.index_copy_(0, real, Sin.index_select(0, last))
     return out
 
 

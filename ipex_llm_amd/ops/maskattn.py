@@ -107,6 +107,10 @@ def qkv_norm_rope_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[
 # portion starts in, whole chunks, the start of a last chunk): pieces of at least GEMM_MIN_CHUNK queries run as
 # batched library products, with the fused softmax (sink, causal mask inside the chunk) between them.
 GEMM_MIN_CHUNK = int(os.environ.get("ILLM_MASKATTN_GEMM_MIN", "128"))
+# Under a sliding window, portions of at least WINDOW_GEMM_MIN queries run the same way in blocks of WINDOW_Q_BLOCK
+# queries: a block's keys are the kept first tokens and everything from its first query's window start on.
+WINDOW_GEMM_MIN = int(os.environ.get("ILLM_MASKATTN_WINDOW_GEMM_MIN", "256"))
+WINDOW_Q_BLOCK = int(os.environ.get("ILLM_MASKATTN_WINDOW_BLOCK", "512"))
 
 
 def masked_attention(q: torch.Tensor, rows: torch.Tensor, G: int, dv: int, block_tables: torch.Tensor,
@@ -183,7 +187,7 @@ def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out
     qq = q[t0:t0 + n].view(nc, nq, G, rep, d).permute(0, 2, 1, 3, 4).reshape(nc * G, nq * rep, d)
     if f32:
         sc = torch.bmm(qq, kk)
-        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, True, softcap, True)
+        w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, True, softcap, True, 0, 0, 0, 0, 0)
         if talk is not None:
             w = _ops().ma_talk_mix(w, talk, nq, G, rep, True)
         o = torch.bmm(w.view(nc * G, nq * rep, nk), vv)
@@ -194,13 +198,58 @@ def _pieces_gemm(q, rows, table_row, G, dv, scale, sink, t0, lo, nc, nk, nq, out
         q2 = torch.cat([qh, (qq - qh.float()).to(rows.dtype)], -1)
         sc = torch.bmm(q2, torch.cat([kk, kk], 1), out_dtype=torch.float32)
         if talk is None:
-            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, False)
+            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, False, 0, 0, 0, 0, 0)
         else:       # normalised f32 weights in place, then the heads' weights mixed and split into hi + lo halves
-            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, True)
+            w = _ops().ma_chunk_softmax(sc.view(nc * G * nq * rep, nk), nq, G, rep, scale, sink, False, softcap, True, 0, 0, 0, 0, 0)
             w = _ops().ma_talk_mix(w, talk, nq, G, rep, False)
         o = torch.bmm(w.view(nc * G, nq * rep, 2 * nk), torch.cat([vv, vv], 1), out_dtype=torch.float32)
     o = o.view(nc, G, nq, rep, dv).permute(0, 2, 1, 3, 4).reshape(n, H * dv)
     out[t0:t0 + n] = o.to(out.dtype)
+
+
+def _window_gemm(q, rows, table_row, G, dv, scale, sink, t0, n, L, size, keep, out, softcap=0.0, talk=None):
+    """A portion of ``n`` queries (the step's tokens from ``t0`` on, the last at position L - 1) of one sequence under
+    a sliding window, block by block of WINDOW_Q_BLOCK queries: a block sees the kept first tokens and the keys from
+    its first query's window start to its last query, as two batched library products per block with the masked
+    softmax between them."""
+    _, H, d = q.shape
+    rep = H // G
+    bs = rows.shape[1]
+    f32 = rows.dtype == torch.float32
+    flat = rows.view(-1, rows.shape[-1])
+    p0 = L - n
+    for b0 in range(0, n, WINDOW_Q_BLOCK):
+        nq = min(WINDOW_Q_BLOCK, n - b0)
+        q0 = p0 + b0
+        k0 = max(0, q0 - size + 1)
+        nkeep = min(keep, k0)
+        nr = q0 + nq - k0
+        nk = -(-(nkeep + nr) // 8) * 8                               # padded columns: masked (ahead of every query)
+        p = torch.cat([torch.arange(nkeep, device=q.device), torch.arange(k0, k0 + nr, device=q.device),
+                       torch.full((nk - nkeep - nr,), k0 + nr - 1, device=q.device)])
+        ridx = table_row.long()[p // bs] * bs + p % bs
+        kv = flat.index_select(0, ridx)
+        kk = kv[:, :G * d].reshape(nk, G, d).permute(1, 2, 0)
+        vv = kv[:, G * d:].reshape(nk, G, dv).permute(1, 0, 2)
+        qq = q[t0 + b0:t0 + b0 + nq].view(nq, G, rep, d).permute(1, 0, 2, 3).reshape(G, nq * rep, d)
+        args = (nq, G, rep, scale, sink, f32, softcap)
+        win = (size, keep, nkeep, q0, k0)
+        if f32:
+            sc = torch.bmm(qq, kk)
+            w = _ops().ma_chunk_softmax(sc.view(G * nq * rep, nk), *args, True, *win)
+            if talk is not None:
+                w = _ops().ma_talk_mix(w, talk, nq, G, rep, True)
+            o = torch.bmm(w.view(G, nq * rep, nk), vv)
+        else:
+            qh = qq.to(rows.dtype)
+            q2 = torch.cat([qh, (qq - qh.float()).to(rows.dtype)], -1)
+            sc = torch.bmm(q2, torch.cat([kk, kk], 1), out_dtype=torch.float32)
+            w = _ops().ma_chunk_softmax(sc.view(G * nq * rep, nk), *args, talk is not None, *win)
+            if talk is not None:
+                w = _ops().ma_talk_mix(w, talk, nq, G, rep, False)
+            o = torch.bmm(w.view(G, nq * rep, 2 * nk), torch.cat([vv, vv], 1), out_dtype=torch.float32)
+        o = o.view(G, nq, rep, dv).permute(1, 0, 2, 3).reshape(nq, H * dv)
+        out[t0 + b0:t0 + b0 + nq] = o.to(out.dtype)
 
 
 def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask, size, sink, q_lens, ctx_lens,
@@ -211,6 +260,25 @@ def _masked_attention_gpu(q, rows, G, dv, block_tables, seq_of, pos, scale, mask
     code = MASKS[mask]
     big = mask == "chunk" and GEMM_MIN_CHUNK > 0 and max(q_lens) >= GEMM_MIN_CHUNK and _bmm_f32_ok(rows.dtype) and \
         (talk is None or H <= 256)
+    if mask == "window" and WINDOW_GEMM_MIN > 0 and max(q_lens) >= WINDOW_GEMM_MIN and _bmm_f32_ok(rows.dtype) and \
+            (talk is None or H <= 256):
+        # long portions run block by block as library products, the others (decoded tokens, short portions) together
+        # through the one-pass kernel
+        out = torch.empty(T, H * dv, dtype=out_dtype, device=q.device)
+        rest, rest_ctx, t0 = [], 1, 0
+        for b, (n, L) in enumerate(zip(q_lens, ctx_lens)):
+            if n >= WINDOW_GEMM_MIN:
+                _window_gemm(q, rows, block_tables[b], G, dv, scale, sink, t0, n, L, size, keep_first, out, softcap, talk)
+            elif n:
+                rest.append(torch.arange(t0, t0 + n, device=q.device))
+                rest_ctx = max(rest_ctx, L)
+            t0 += n
+        if rest:
+            idx = torch.cat(rest)
+            out[idx] = _ops().ma_masked_attention(q[idx].contiguous(), rows, G, dv, block_tables,
+                                                  seq_of[idx].contiguous(), pos[idx].contiguous(), scale, code, size, sink,
+                                                  rest_ctx, f32, softcap, keep_first, talk)
+        return out
     if not big:
         return _ops().ma_masked_attention(q, rows, G, dv, block_tables, seq_of, pos, scale, code, size, sink,
                                           max(ctx_lens), f32, softcap, keep_first, talk)

@@ -242,6 +242,32 @@ def test_gla_scan_op(dev, H, d, dv):
             assert (o - want).abs().max() < 2e-4 * max(1.0, float(want.abs().max()))
 
 
+def test_gla_long_portions_run_in_pieces(dev):
+    """portions long enough to be cut into pieces that run side by side on the GPU (each piece's start state comes
+    from the chain of the pieces before it), beside a short one; a fresh sequence and one that continues"""
+    from ipex_llm_amd.ops import gatedmix as GM
+    g = torch.Generator().manual_seed(5)
+    H, d, dv, tau = 2, 16, 8, 6.0
+    lens, starts = [2100, 5, 1300], [0, 3, 70]
+    T = sum(lens)
+    q, k = torch.randn(T, H, d, generator=g), torch.randn(T, H, d, generator=g)
+    v, a = torch.randn(T, H, dv, generator=g), torch.randn(T, H, d, generator=g) * 2 + 3
+    S0 = torch.randn(6, H, d, dv, generator=g)
+    state = S0.clone().to(dev)
+    cu, _, slots, pos = ragged(lens, starts, dev)
+    got = GM.gla_scan(q.to(dev), k.to(dev), v.to(dev), a.to(dev), tau, 0.25, state, cu, slots, pos, lens).double().cpu()
+    alpha = O.sigmoid(a.double()) ** (1 / tau)
+    t0 = 0
+    for s, n in enumerate(lens):
+        S = torch.zeros(H, d, dv, dtype=F64) if starts[s] == 0 else S0[s + 1].double()
+        for t in range(t0, t0 + n):
+            S = alpha[t][:, :, None] * S + k[t].double()[:, :, None] * v[t].double()[:, None, :]
+            want = (S * (q[t].double() * 0.25)[:, :, None]).sum(1)
+            assert (got[t] - want).abs().max() < 2e-4 * max(1.0, float(want.abs().max())), (s, t - t0)
+        assert (state[s + 1].double().cpu() - S).abs().max() < 2e-4 * max(1.0, float(S.abs().max()))
+        t0 += n
+
+
 def test_head_norm_pair_mean_and_cap(dev):
     from ipex_llm_amd.ops import gatedmix as GM
     g = torch.Generator().manual_seed(1)
@@ -582,6 +608,21 @@ def test_long_chunks_take_the_product_path(dev, chunk, sizes):
     for dtype in (torch.float32, torch.bfloat16):
         got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", n)] for n in sizes])["a"]
         assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("window,keep,sizes", [(100, 3, [50, 390, 10]), (300, 40, [300, 150]), (64, 0, [5, 445]), (700, 9, [450])])
+def test_long_windows_take_the_product_path(dev, window, keep, sizes):
+    """portions long enough for the block-by-block product path of a sliding window on the GPU: blocks whose window
+    starts before, at and after the kept first tokens, a portion that continues what an earlier step left"""
+    cfg = O.config([O.pair_layer(heads=4, kv_heads=2, dim=16, vdim=24, window=window, keep=keep, taps=2, dims=8,
+                                 mlp=O.moe(3, 2, 8)), O.gru_layer(width=8)], width=32)
+    W = O.random_weights(cfg, 17)
+    toks = O.random_tokens(cfg, 450, 17)
+    want = oracle(cfg, W, toks, f"w{window}")
+    for dtype in (torch.float32, torch.bfloat16):
+        got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", n)] for n in sizes])["a"]
+        # 16-bit: the worst of 450 rows behind two recurrences and up to 340 keys in view
+        assert rel_err(got, want) < (TOL[dtype] if dtype == torch.float32 else 0.3)
 
 
 def test_greedy_generation_scheduler(dev):
