@@ -167,7 +167,7 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_pre: torch.Ten
 # that run side by side, twice: the recurrence is linear in the state, S_end = diag(P) S_start + Z with P the product
 # of the piece's decays and Z its result from a zero state, so a first pass gives every piece's Z, a short chain
 # over the pieces gives every piece's true start state, and a second pass from those writes the outputs.
-GLA_PIECE_MIN = int(os.environ.get("ILLM_GLA_PIECE_MIN", "1024"))
+GLA_PIECE_MIN = int(os.environ.get("ILLM_GLA_PIECE_MIN", "2048"))
 GLA_PIECES = int(os.environ.get("ILLM_GLA_PIECES", "16"))
 
 

@@ -109,7 +109,7 @@ def qkv_norm_rope_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[
 GEMM_MIN_CHUNK = int(os.environ.get("ILLM_MASKATTN_GEMM_MIN", "128"))
 # Under a sliding window, portions of at least WINDOW_GEMM_MIN queries run the same way in blocks of WINDOW_Q_BLOCK
 # queries: a block's keys are the kept first tokens and everything from its first query's window start on.
-WINDOW_GEMM_MIN = int(os.environ.get("ILLM_MASKATTN_WINDOW_GEMM_MIN", "256"))
+WINDOW_GEMM_MIN = int(os.environ.get("ILLM_MASKATTN_WINDOW_GEMM_MIN", "1536"))
 WINDOW_Q_BLOCK = int(os.environ.get("ILLM_MASKATTN_WINDOW_BLOCK", "512"))
 
 
