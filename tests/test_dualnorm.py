@@ -242,10 +242,11 @@ def test_gla_scan_op(dev, H, d, dv):
             assert (o - want).abs().max() < 2e-4 * max(1.0, float(want.abs().max()))
 
 
-def test_gla_long_portions_run_in_pieces(dev):
+def test_gla_long_portions_run_in_pieces(dev, monkeypatch):
     """portions long enough to be cut into pieces that run side by side on the GPU (each piece's start state comes
     from the chain of the pieces before it), beside a short one; a fresh sequence and one that continues"""
     from ipex_llm_amd.ops import gatedmix as GM
+    monkeypatch.setattr(GM, "GLA_PIECE_MIN", 1024)
     g = torch.Generator().manual_seed(5)
     H, d, dv, tau = 2, 16, 8, 6.0
     lens, starts = [2100, 5, 1300], [0, 3, 70]
@@ -611,9 +612,13 @@ def test_long_chunks_take_the_product_path(dev, chunk, sizes):
 
 
 @pytest.mark.parametrize("window,keep,sizes", [(100, 3, [50, 390, 10]), (300, 40, [300, 150]), (64, 0, [5, 445]), (700, 9, [450])])
-def test_long_windows_take_the_product_path(dev, window, keep, sizes):
-    """portions long enough for the block-by-block product path of a sliding window on the GPU: blocks whose window
-    starts before, at and after the kept first tokens, a portion that continues what an earlier step left"""
+def test_long_windows_take_the_product_path(dev, window, keep, sizes, monkeypatch):
+    """portions long enough for the block-by-block product path of a sliding window on the GPU (its threshold and
+    block lowered to this test's lengths): blocks whose window starts before, at and after the kept first tokens, a
+    portion that continues what an earlier step left"""
+    from ipex_llm_amd.ops import maskattn as MA
+    monkeypatch.setattr(MA, "WINDOW_GEMM_MIN", 128)
+    monkeypatch.setattr(MA, "WINDOW_Q_BLOCK", 160)
     cfg = O.config([O.pair_layer(heads=4, kv_heads=2, dim=16, vdim=24, window=window, keep=keep, taps=2, dims=8,
                                  mlp=O.moe(3, 2, 8)), O.gru_layer(width=8)], width=32)
     W = O.random_weights(cfg, 17)
