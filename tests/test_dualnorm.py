@@ -496,6 +496,21 @@ def test_small_models_bf16(dev, case):
     assert rel_err(got, O.forward(cfg, W, toks)) < TOL[torch.bfloat16]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_odd_sizes(dev, dtype):
+    """widths, head sizes, expert sizes, side size and vocabulary that are multiples of nothing"""
+    cfg = O.config([O.attn_layer(heads=3, kv_heads=1, dim=9, vdim=7, chunk=5, taps=3, mlp=O.moe(3, 2, 5)),
+                    O.gru_layer(width=11, mlp=O.moe(2, 1, 7)),
+                    O.attn_layer(heads=3, kv_heads=1, dim=9, vdim=7, chunk=5, taps=2, kv_from=0),
+                    O.pair_layer(heads=5, kv_heads=5, dim=9, vdim=3, window=6, keep=1, taps=3, dims=4, rheads=3, rdim=5,
+                                 rvdim=3, tau=2.5, mlp=O.moe(5, 5, 3))], vocab=53, width=37, side=5)
+    W = O.random_weights(cfg, 31)
+    toks = O.random_tokens(cfg, 70, 31)
+    got = replay(engine(cfg, W, dev, dtype), {"a": toks}, [[("a", 33)], [("a", 30)]] + [[("a", 1)]] * 7)["a"]
+    # 16-bit: rows of 3 to 37 values average little rounding away
+    assert rel_err(got, O.forward(cfg, W, toks)) < (TOL[dtype] if dtype == torch.float32 else 0.2)
+
+
 def test_whole_prompt_and_layers(dev):
     cfg = std_cfg()
     W = O.random_weights(cfg, 7)
