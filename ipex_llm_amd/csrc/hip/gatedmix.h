@@ -30,6 +30,14 @@ void gla_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_l
               const void* a, int64_t a_ld, float tau, float q_scale, float* S, const int32_t* cu, const int32_t* slots,
               const int64_t* pos, float* out, int B, int H, int d, int dv, hipStream_t st);
 
+// a long portion cut into pieces that run side by side: P f32 [NP, H, d] = the product of every piece's decays
+// (cu int32 [NP + 1]: the pieces' token borders), and the chain of the pieces' start states: Z / Sin f32
+// [NP + 1, H, d, dv] (Z: every piece's end state from the first pass), seqs int32 [nseq, 2] = first piece, pieces
+void gla_piece_decay(bool bf16, const void* a, int64_t a_ld, const int32_t* cu, float tau, float* P, int NP, int H, int d,
+                     hipStream_t st);
+void gla_chain(const float* Z, float* Sin, const float* P, const int32_t* seqs, int nseq, int H, int d, int dv,
+               hipStream_t st);
+
 // o f32 [T, H, dv]; w [dv]; gate rows of g_ld elements; out [T, H dv]
 void head_rms_silu(bool bf16, const float* o, const void* w, const void* gate, int64_t g_ld, void* out, int T, int H,
                    int dv, float eps, hipStream_t st);

@@ -292,6 +292,51 @@ __global__ void __launch_bounds__(MAXT) gla_scan_k(const E* __restrict__ q, int6
   }
 }
 
+// the product of a piece's decays per (head, key channel): P = exp(sum_t log_sigmoid(a_t) / tau), summed in f64.
+// One workgroup per (piece, head): 64 channels x 4 token groups
+template <typename E>
+__global__ void __launch_bounds__(256) gla_piece_decay_k(const E* __restrict__ a, int64_t a_ld,
+                                                        const int32_t* __restrict__ cu, float inv_tau,
+                                                        float* __restrict__ P, int H, int d) {
+  __shared__ double part[4][64];
+  const int piece = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, tg = threadIdx.x >> 6;
+  const int t0 = cu[piece], t1 = cu[piece + 1];
+  for (int r0 = 0; r0 < d; r0 += 64) {
+    const int r = r0 + lane;
+    double sum = 0.0;
+    if (r < d)
+      for (int t = t0 + tg; t < t1; t += 4) {
+        const float z = ldf(a + (int64_t)t * a_ld + h * d + r);
+        sum += (double)(fminf(z, 0.f) - log1pf(expf(-fabsf(z))));
+      }
+    __syncthreads();
+    part[tg][lane] = sum;
+    __syncthreads();
+    if (tg == 0 && r < d)
+      P[((int64_t)piece * H + h) * d + r] =
+          expf((float)((part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]) * (double)inv_tau));
+  }
+}
+
+// start states of the pieces of a sequence, piece after piece: the first piece's end state Z[f] starts the second;
+// then S <- diag(P) S + Z.  seqs int32 [n][2]: first piece, number of pieces
+__global__ void __launch_bounds__(256) gla_chain_k(const float* __restrict__ Z, float* __restrict__ Sin,
+                                                  const float* __restrict__ P, const int32_t* __restrict__ seqs, int HD,
+                                                  int dv) {
+  const int f = seqs[2 * blockIdx.x], m = seqs[2 * blockIdx.x + 1];
+  if (m < 2) return;
+  const int64_t n = (int64_t)HD * dv;
+  for (int64_t e = (int64_t)blockIdx.y * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.y * blockDim.x) {
+    const int64_t hr = e / dv;
+    float S = Z[f * n + e];
+    Sin[(f + 1) * n + e] = S;
+    for (int j = 2; j < m; j++) {
+      S = fmaf(P[(int64_t)(f + j - 1) * HD + hr], S, Z[(f + j - 1) * n + e]);
+      Sin[(f + j) * n + e] = S;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ element-wise steps
 template <typename E>
 __global__ void __launch_bounds__(64) head_rms_silu_k(const float* __restrict__ o, const E* __restrict__ nw,
@@ -397,6 +442,21 @@ void gla_scan(bool bf16, const void* q, int64_t q_ld, const void* k, int64_t k_l
 #undef GM_GLA_NS
 #undef GM_GLA
 #undef GM_GLA_T
+}
+
+void gla_piece_decay(bool bf16, const void* a, int64_t a_ld, const int32_t* cu, float tau, float* P, int NP, int H, int d,
+                     hipStream_t st) {
+  if (NP <= 0) return;
+  if (bf16) gla_piece_decay_k<__bf16><<<dim3(NP, H), 256, 0, st>>>((const __bf16*)a, a_ld, cu, 1.0f / tau, P, H, d);
+  else gla_piece_decay_k<float><<<dim3(NP, H), 256, 0, st>>>((const float*)a, a_ld, cu, 1.0f / tau, P, H, d);
+}
+
+void gla_chain(const float* Z, float* Sin, const float* P, const int32_t* seqs, int nseq, int H, int d, int dv,
+               hipStream_t st) {
+  if (nseq <= 0) return;
+  const int64_t n = (int64_t)H * d * dv;
+  const int by = (int)((n + 255) / 256 > 1024 ? 1024 : (n + 255) / 256);
+  gla_chain_k<<<dim3(nseq, by), 256, 0, st>>>(Z, Sin, P, seqs, H * d, dv);
 }
 
 void head_rms_silu(bool bf16, const float* o, const void* w, const void* gate, int64_t g_ld, void* out, int T, int H,

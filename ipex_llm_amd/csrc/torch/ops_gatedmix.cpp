@@ -124,6 +124,36 @@ Tensor gm_gla_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tens
   return out;
 }
 
+Tensor gm_gla_piece_decay(const Tensor& a, const Tensor& cu, double tau) {
+  c10::DeviceGuard g(a.device());
+  TORCH_CHECK(is_act(a) && head_rows(a, a.scalar_type()), "gm_gla_piece_decay: a [T, H, d] (heads contiguous in a row)");
+  TORCH_CHECK(cu.is_cuda() && cu.scalar_type() == at::kInt && cu.is_contiguous() && cu.numel() >= 2 && tau > 0,
+              "gm_gla_piece_decay: cu int32 [NP + 1], tau > 0");
+  const int64_t NP = cu.numel() - 1, H = a.size(1), d = a.size(2);
+  TORCH_CHECK(H <= 65535, "gm_gla_piece_decay: too many heads for one launch");
+  Tensor P = at::empty({NP, H, d}, a.options().dtype(at::kFloat));
+  illm::gm::gla_piece_decay(bf(a), a.data_ptr(), a.stride(0), cu.data_ptr<int32_t>(), (float)tau, P.data_ptr<float>(),
+                            (int)NP, (int)H, (int)d, stream());
+  return P;
+}
+
+void gm_gla_chain_(const Tensor& Z, Tensor& Sin, const Tensor& P, const Tensor& seqs) {
+  c10::DeviceGuard g(Z.device());
+  TORCH_CHECK(Z.is_cuda() && Z.scalar_type() == at::kFloat && Z.is_contiguous() && Z.dim() == 4,
+              "gm_gla_chain_: Z f32 [pieces + 1, H, d, dv]");
+  TORCH_CHECK(Sin.is_cuda() && Sin.scalar_type() == at::kFloat && Sin.is_contiguous() && Sin.sizes() == Z.sizes(),
+              "gm_gla_chain_: Sin like Z");
+  const int64_t H = Z.size(1), d = Z.size(2), dv = Z.size(3);
+  TORCH_CHECK(P.is_cuda() && P.scalar_type() == at::kFloat && P.is_contiguous() && P.dim() == 3 &&
+                  P.size(0) + 1 == Z.size(0) && P.size(1) == H && P.size(2) == d,
+              "gm_gla_chain_: P f32 [pieces, H, d]");
+  TORCH_CHECK(seqs.is_cuda() && seqs.scalar_type() == at::kInt && seqs.is_contiguous() && seqs.dim() == 2 &&
+                  seqs.size(1) == 2 && seqs.size(0) <= 65535,
+              "gm_gla_chain_: seqs int32 [n, 2]");
+  illm::gm::gla_chain(Z.data_ptr<float>(), Sin.data_ptr<float>(), P.data_ptr<float>(), seqs.data_ptr<int32_t>(),
+                      (int)seqs.size(0), (int)H, (int)d, (int)dv, stream());
+}
+
 Tensor gm_head_rms_silu(const Tensor& o, const Tensor& w, const Tensor& gate, double eps, bool act_f32) {
   c10::DeviceGuard g(o.device());
   TORCH_CHECK(o.is_cuda() && o.dim() == 3 && o.scalar_type() == at::kFloat && o.is_contiguous(),
@@ -172,6 +202,8 @@ TORCH_LIBRARY_FRAGMENT(ipex_llm_amd, m) {
   m.def("gm_mingru_scan(Tensor y, int width, Tensor(a!) state, Tensor cu, Tensor slots, Tensor pos, int max_n) -> Tensor");
   m.def("gm_gla_scan(Tensor q, Tensor k, Tensor v, Tensor a, float tau, float q_scale, Tensor(a!) S, Tensor cu, "
         "Tensor slots, Tensor pos) -> Tensor");
+  m.def("gm_gla_piece_decay(Tensor a, Tensor cu, float tau) -> Tensor");
+  m.def("gm_gla_chain_(Tensor Z, Tensor(a!) Sin, Tensor P, Tensor seqs) -> ()");
   m.def("gm_head_rms_silu(Tensor o, Tensor w, Tensor gate, float eps, bool act_f32) -> Tensor");
   m.def("gm_rms_pair_mean(Tensor a, Tensor b, Tensor wa, Tensor wb, float eps, bool act_f32) -> Tensor");
   m.def("gm_softcap_(Tensor(a!) x, float cap) -> Tensor(a!)");
@@ -181,6 +213,8 @@ TORCH_LIBRARY_IMPL(ipex_llm_amd, CUDA, m) {
   m.impl("gm_layer_norm_pair_shift", &gm_layer_norm_pair_shift);
   m.impl("gm_mingru_scan", &gm_mingru_scan);
   m.impl("gm_gla_scan", &gm_gla_scan);
+  m.impl("gm_gla_piece_decay", &gm_gla_piece_decay);
+  m.impl("gm_gla_chain_", &gm_gla_chain_);
   m.impl("gm_head_rms_silu", &gm_head_rms_silu);
   m.impl("gm_rms_pair_mean", &gm_rms_pair_mean);
   m.impl("gm_softcap_", &gm_softcap_);

@@ -348,8 +348,9 @@ def moe_route(z: torch.Tensor, top: int, mode: str = "sigmoid") -> Tuple[torch.T
     logits only."""
     if mode not in ROUTE_MODES:
         raise ValueError(f"unknown router mode {mode!r}")
-    if native(z):
+    if native(z) and z.shape[1] <= 512 and (mode == "sigmoid" or top <= 64):
         return _ops().bm_moe_route(z.contiguous(), top, ROUTE_MODES[mode])
+    # (sizes past the kernel's: library sort)
     val, idx = torch.sort(z.float(), dim=-1, descending=True, stable=True)
     val = val[:, :top]
     w = torch.sigmoid(val) if mode == "sigmoid" else torch.softmax(val, -1)

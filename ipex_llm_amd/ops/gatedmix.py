@@ -174,7 +174,7 @@ GLA_PIECES = int(os.environ.get("ILLM_GLA_PIECES", "16"))
 def _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_lens):
     T, H, d = q.shape
     dev = q.device
-    cuts, first, owner, spans = [0], [], [], []      # piece borders (token indices); first piece of / pieces per sequence
+    cuts, first, owner = [0], [], []                 # piece borders (token indices); first piece of / pieces per sequence
     t0 = 0
     for s, n in enumerate(q_lens):
         if n == 0:
@@ -184,7 +184,6 @@ def _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_le
         for lo in range(0, n, per):
             cuts.append(t0 + min(n, lo + per))
         owner.append((s, len(cuts) - 1 - first[-1]))
-        spans.append((t0, n, per))
         t0 += n
     NP = len(cuts) - 1
     cu_p = torch.tensor(cuts, dtype=torch.int32, device=dev)
@@ -193,13 +192,9 @@ def _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_le
     seqs = torch.tensor([s for s, _ in owner], dtype=torch.long, device=dev)
     real = state_slots.long().index_select(0, seqs)
     later = torch.tensor([cuts[f + j] for f, (_, m) in zip(first, owner) for j in range(1, m)], dtype=torch.long, device=dev)
-    # every piece's decay product (of the sequences that have several pieces): sums of log decays in f64
-    P = {}
-    for f, (_, m), (s0, n, per) in zip(first, owner, spans):
-        if m > 1:
-            ls = F.logsigmoid(a_pre[s0:s0 + n].float())
-            ls = F.pad(ls, (0, 0, 0, 0, 0, m * per - n)).view(m, per, H, d).double().sum(1)
-            P[f] = torch.exp(ls / tau).float()                          # [m, H, d]
+    # every piece's decay product (sums of log decays in f64)
+    P = _ops().gm_gla_piece_decay(a_pre, cu_p, tau)                     # [NP, H, d]
+    seqs_p = torch.tensor([[f, m] for f, (_, m) in zip(first, owner)], dtype=torch.int32, device=dev)
     start = state.index_select(0, real)
     Z = torch.empty(NP + 1, *state.shape[1:], dtype=torch.float32, device=dev)
     Z.index_copy_(0, first_t, start)
@@ -208,12 +203,7 @@ def _gla_scan_pieces(q, k, v, a_pre, tau, q_scale, state, state_slots, pos, q_le
     _ops().gm_gla_scan(q, k, v, a_pre, tau, q_scale, Z, cu_p, slots_p, pos1)
     Sin = torch.empty_like(Z)
     Sin.index_copy_(0, first_t, start)
-    for f, (_, m) in zip(first, owner):                                 # the chain of start states, piece after piece
-        for j in range(1, m):
-            if j == 1:
-                Sin[f + 1].copy_(Z[f])                                  # the first piece's Z holds its start state too
-            else:
-                torch.addcmul(Z[f + j - 1], Sin[f + j - 1], P[f][j - 1].unsqueeze(-1), out=Sin[f + j])
+    _ops().gm_gla_chain_(Z, Sin, P, seqs_p)                             # the chain of start states, piece after piece
     out = _ops().gm_gla_scan(q, k, v, a_pre, tau, q_scale, Sin, cu_p, slots_p, pos)
     last = torch.tensor([f + m - 1 for f, (_, m) in zip(first, owner)], dtype=torch.long, device=dev)
     state.index_copy_(0, real, Sin.index_select(0, last))
